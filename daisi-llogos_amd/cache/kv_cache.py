@@ -31,10 +31,11 @@ class KVGroup:
             # hands out: the page of padding rows (Cache.pad_page)
             shape = (len(entries), n_pages + 1, spec.n_kv_heads, PAGE_TOKENS * spec.head_dim)
             self.k = torch.zeros(shape, dtype=rt.dtype, device=rt.device)
-            self.v = torch.zeros(shape, dtype=rt.dtype, device=rt.device)
+            if spec.values:                  # (a latent cache has key rows only)
+                self.v = torch.zeros(shape, dtype=rt.dtype, device=rt.device)
 
     def bytes(self) -> int:
-        return 0 if self.k is None else 2 * self.k.numel() * self.k.element_size()
+        return 0 if self.k is None else (2 if self.v is not None else 1) * self.k.numel() * self.k.element_size()
 
 
 class Cache:
@@ -131,7 +132,7 @@ class Cache:
         if self.rt is None:
             return 0
         elt = torch.empty((), dtype=self.rt.dtype).element_size()
-        return sum(2 * len(g.entries) * g.spec.n_kv_heads * g.spec.head_dim * elt for g in self.groups)
+        return sum((2 if g.spec.values else 1) * len(g.entries) * g.spec.n_kv_heads * g.spec.head_dim * elt for g in self.groups)
 
     # ---- a step's storage ----------------------------------------------------------
     def reserve(self, slot_ids: Sequence[int], new_lens: Sequence[int]) -> None:
@@ -197,7 +198,7 @@ class Cache:
             if loc is not None:
                 g, i = loc
                 grp = self.groups[g]
-                lc.k_pool, lc.v_pool, lc.table = grp.k[i], grp.v[i], tables[g]
+                lc.k_pool, lc.v_pool, lc.table = grp.k[i], (grp.v[i] if grp.v is not None else None), tables[g]
                 lc.writes = self.reads_from[e] is None or self.reads_from[e] == e
             out.append(lc)
         return out

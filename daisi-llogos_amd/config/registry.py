@@ -16,22 +16,26 @@ from .model_config import ConfigError, DenseDecoderConfig
 @dataclass(frozen=True)
 class Architecture:
     name: str
-    read_config: Callable[[dict], object]        # parsed config.json -> typed configuration
+    read_config: Callable[..., object]           # parsed config.json -> typed configuration
     model_spec: Callable[..., object]            # typed configuration (+ options) -> ModelSpec
+    reads_shapes: bool = False                   # read_config also takes shapes={tensor name: shape} of the checkpoint,
+                                                 # for sizes that the file leaves to the tensors
 
 
 ARCHITECTURES: Dict[str, Architecture] = {}
 
 
-def register_architecture(name: str, read_config: Callable[[dict], object],
-                          model_spec: Callable[..., object]) -> Architecture:
-    arch = Architecture(name, read_config, model_spec)
+def register_architecture(name: str, read_config: Callable[..., object],
+                          model_spec: Callable[..., object], reads_shapes: bool = False) -> Architecture:
+    arch = Architecture(name, read_config, model_spec, reads_shapes)
     ARCHITECTURES[name] = arch
     return arch
 
 
 def architecture_of(data: dict) -> Architecture:
     archs = data.get("architectures") if isinstance(data, dict) else None
+    if archs is None and isinstance(data, dict) and isinstance(data.get("architecture"), str):
+        archs = [data["architecture"]]               # files that name one design in a string
     if not isinstance(archs, list) or not archs or not isinstance(archs[0], str):
         raise ConfigError("config.json: missing key 'architectures' (a list with the model's class name)")
     name = archs[0]
@@ -51,3 +55,12 @@ def _dense(name: str, bias_default: bool, qk_norm: bool) -> None:
 _dense("LlamaForCausalLM", bias_default=False, qk_norm=False)
 _dense("Qwen2ForCausalLM", bias_default=True, qk_norm=False)
 _dense("Qwen3ForCausalLM", bias_default=False, qk_norm=True)
+
+
+def _nipulorn() -> None:
+    from ..models.nipulorn import nipulorn_spec
+    from .nipulorn_config import NipulornConfig
+    register_architecture("Nipulorn", NipulornConfig.from_dict, nipulorn_spec, reads_shapes=True)
+
+
+_nipulorn()

@@ -4,6 +4,10 @@
 // in tiles of 256 that start at key 0, with a running maximum and sum, so the order of
 // the additions for a query depends on its position alone and not on how the tokens
 // were cut into steps or on what else is in the batch.
+// Two options serve mixers whose cache differs from keys and values of one size:
+//   v_dim < head_dim with no value pool: a value is the first v_dim dimensions of its key row;
+//   head_sink [n_heads]: the softmax's denominator also holds exp(head_sink[h]), a learned score
+//   without a key or a value (the running maximum and sum start from it).
 // (reference: gated_attention / batched_gated_attention,
 //  Daisi.Llogos.Cuda/kernels/composite_ops.cu:275-387, 396-512: kv head = head / group,
 //  scale after the dot, tiles of 256 keys, running max and sum; the sigmoid gate of that
@@ -11,14 +15,15 @@
 #include "common.h"
 
 constexpr int kTileKeys = 256;
-constexpr int kMaxHeadDimGeneric = 512;
+constexpr int kMaxHeadDimGeneric = 1024;
 
 template <typename T>
 __global__ __launch_bounds__(256) void attn_generic_kernel(
         T* __restrict__ out, const T* __restrict__ q, int q_stride,
         const T* __restrict__ k_pool, const T* __restrict__ v_pool, PagedKV cache,
         const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
-        int n_heads, int group, int head_dim, float scale, int window, int sinks) {
+        int n_heads, int group, int head_dim, float scale, int window, int sinks,
+        int v_dim, const float* __restrict__ head_sink) {
     extern __shared__ float smem[];
     float* qf = smem;                    // [head_dim]
     float* p_lds = smem + head_dim;      // [kTileKeys]
@@ -32,6 +37,7 @@ __global__ __launch_bounds__(256) void attn_generic_kernel(
     __syncthreads();
 
     float m_run = -INFINITY, l_run = 0.f;
+    if (head_sink) { m_run = head_sink[h]; l_run = 1.f; }
     float acc[kMaxHeadDimGeneric / 256] = {};
 
     for (int j0 = 0; j0 <= pos; j0 += kTileKeys) {
@@ -58,13 +64,16 @@ __global__ __launch_bounds__(256) void attn_generic_kernel(
 #pragma unroll
         for (int r = 0; r < kMaxHeadDimGeneric / 256; ++r) {
             const int d = tid + r * 256;
-            if (d < head_dim) {
+            if (d < v_dim) {
                 float a = acc[r] * corr;
                 for (int jj = 0; jj < n_keys; ++jj) {
                     const float pj = p_lds[jj];
-                    if (pj != 0.f)
-                        a = fmaf(pj, load_f32(v_pool + paged_base(cache, seq, kvh, j0 + jj)
-                                              + page_value_offset((j0 + jj) % kPageTokens, d)), a);
+                    if (pj != 0.f) {
+                        const size_t base = paged_base(cache, seq, kvh, j0 + jj);
+                        const int tk = (j0 + jj) % kPageTokens;
+                        a = fmaf(pj, v_pool ? load_f32(v_pool + base + page_value_offset(tk, d))
+                                            : load_f32(k_pool + base + page_key_offset(tk, d, head_dim)), a);
+                    }
                 }
                 acc[r] = a;
             }
@@ -73,11 +82,11 @@ __global__ __launch_bounds__(256) void attn_generic_kernel(
         m_run = m_new;
     }
     const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
-    T* orow = out + ((size_t)t * n_heads + h) * head_dim;
+    T* orow = out + ((size_t)t * n_heads + h) * v_dim;
 #pragma unroll
     for (int r = 0; r < kMaxHeadDimGeneric / 256; ++r) {
         const int d = tid + r * 256;
-        if (d < head_dim) store_f32(orow + d, acc[r] * inv);
+        if (d < v_dim) store_f32(orow + d, acc[r] * inv);
     }
 }
 
@@ -86,7 +95,9 @@ LLOGOS_EXPORT int llogos_attention_generic(void* out, const void* q, int dtype, 
                                            const int* table, int table_stride,
                                            const int* tok_seq, const int* tok_pos,
                                            int T, int n_heads, int n_kv_heads, int head_dim,
-                                           float scale, int window, int sinks, hipStream_t stream) {
+                                           float scale, int window, int sinks, int v_dim, const float* head_sink,
+                                           hipStream_t stream) {
+    if (v_dim <= 0 || v_dim > head_dim || (!v_pool && !k_pool)) return LLOGOS_BAD_ARGUMENT;
     if (T <= 0 || n_heads <= 0 || n_kv_heads <= 0 || n_heads % n_kv_heads != 0) return LLOGOS_BAD_ARGUMENT;
     if (head_dim <= 0 || head_dim > kMaxHeadDimGeneric || window < 0 || sinks < 0) return LLOGOS_BAD_ARGUMENT;
     PagedKV cache{table, table_stride, n_kv_heads, head_dim};
@@ -96,11 +107,11 @@ LLOGOS_EXPORT int llogos_attention_generic(void* out, const void* q, int dtype, 
     if (dtype == DT_F32)
         attn_generic_kernel<float><<<grid, 256, smem, stream>>>(
             (float*)out, (const float*)q, q_stride, (const float*)k_pool, (const float*)v_pool, cache,
-            tok_seq, tok_pos, n_heads, group, head_dim, scale, window, sinks);
+            tok_seq, tok_pos, n_heads, group, head_dim, scale, window, sinks, v_dim, head_sink);
     else if (dtype == DT_BF16)
         attn_generic_kernel<bf16_t><<<grid, 256, smem, stream>>>(
             (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, cache,
-            tok_seq, tok_pos, n_heads, group, head_dim, scale, window, sinks);
+            tok_seq, tok_pos, n_heads, group, head_dim, scale, window, sinks, v_dim, head_sink);
     else
         return LLOGOS_BAD_ARGUMENT;
     return LLOGOS_LAUNCH_CHECK();

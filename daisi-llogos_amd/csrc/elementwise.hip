@@ -250,19 +250,21 @@ LLOGOS_EXPORT int llogos_residual_add(float* x, const void* delta, int delta_dty
 // (reference: Daisi.Llogos.Cpu/Rope.cs:147-152; Daisi.Llogos.Cuda/kernels/elementwise.cu:258-261).
 // One table serves every layer that shares the rotary parameters.
 __global__ void rope_table_kernel(float2* __restrict__ cs, const int* __restrict__ pos,
-                                  const double* __restrict__ inv_freq, int T, int half) {
+                                  const double* __restrict__ inv_freq, int T, int half, double amplitude) {
     const int idx = blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= T * half) return;
     const int t = idx / half, i = idx % half;
     const double a = (double)pos[t] * inv_freq[i];
-    cs[idx] = make_float2((float)cos(a), (float)sin(a));
+    cs[idx] = make_float2((float)(cos(a) * amplitude), (float)(sin(a) * amplitude));
 }
 
+// amplitude multiplies both entries (1 for a plain rotation; scaling rules for long contexts
+// stretch the rotated vectors a little).
 LLOGOS_EXPORT int llogos_rope_table(void* cs, const int* pos, const double* inv_freq, int T, int half,
-                                    hipStream_t stream) {
+                                    double amplitude, hipStream_t stream) {
     if (T <= 0 || half <= 0) return LLOGOS_BAD_ARGUMENT;
     const int n = T * half;
-    rope_table_kernel<<<(n + 255) / 256, 256, 0, stream>>>((float2*)cs, pos, inv_freq, T, half);
+    rope_table_kernel<<<(n + 255) / 256, 256, 0, stream>>>((float2*)cs, pos, inv_freq, T, half, amplitude);
     return LLOGOS_LAUNCH_CHECK();
 }
 

@@ -1,0 +1,145 @@
+// Attention through a low-rank latent.  Each token leaves one vector in the cache,
+//     key row = [ c (rank) | rotated shared key part (rot) | zeros up to the page's head size ],
+// with c the normed latent; there is one such row for all heads and no value pool: a value
+// is the first `rank` dimensions of the key row.  Queries are brought into the same space
+// (q_h . W_uk,h for the unrotated part, the rotated part as it is), so a head's score is one
+// dot product with the cached row, and a head's output is a weighted sum of latents that the
+// value matrix W_uv,h is applied to afterwards.
+#include "common.h"
+
+// ---------------------------------------------------------------- latent norm, rotation, cache write
+// One block per token.  kv [T, ldkv] float: the first `rank` values are RMS-normed with weight
+// norm_w (as it is) and stored as dimensions 0..rank-1 of the token's key row; the next `rot`
+// are the shared key part: its first rot_dims dimensions are rotated in neighbouring pairs
+// (2i, 2i + 1) by the table cs [T, rot_dims / 2] of (cos, sin), the rest pass unchanged.
+// qfull [T, ldq] float holds per head [dim | rot]; the head's rot part is rotated the same way
+// and written to q_out[t, h, rank .. rank + rot), zeros behind it up to hd.
+template <typename T>
+__global__ void latent_prepare_kernel(const float* __restrict__ kv, int ldkv, const float* __restrict__ qfull, int ldq,
+                                      T* __restrict__ q_out, const float* __restrict__ norm_w, float eps,
+                                      const float2* __restrict__ cs, T* __restrict__ k_pool, PagedKV cache,
+                                      const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
+                                      int n_heads, int dim, int rot, int rot_dims, int rank, int hd) {
+    __shared__ float red[16];
+    const int t = blockIdx.x, tid = threadIdx.x;
+    const int seq = tok_seq[t], pos = tok_pos[t];
+    const float* row = kv + (size_t)t * ldkv;
+    const int half = rot_dims / 2;
+    const float2* tab = cs + (size_t)t * half;
+    T* page = k_pool + paged_base(cache, seq, 0, pos);
+    const int in_page = pos % kPageTokens;
+
+    float ss = 0.f;
+    for (int i = tid; i < rank; i += blockDim.x) ss = fmaf(row[i], row[i], ss);
+    const float inv = 1.0f / sqrtf(block_sum(ss, red) / (float)rank + eps);
+    for (int i = tid; i < rank; i += blockDim.x)
+        store_f32(page + page_key_offset(in_page, i, hd), row[i] * inv * norm_w[i]);
+    for (int i = tid; i < hd - rank; i += blockDim.x) {
+        float v = 0.f;
+        if (i < rot) {
+            v = row[rank + i];
+            if (i < rot_dims) {
+                const float2 c = tab[i >> 1];
+                const float other = row[rank + (i ^ 1)];
+                v = (i & 1) ? fmaf(v, c.x, other * c.y) : fmaf(v, c.x, -other * c.y);
+            }
+        }
+        store_f32(page + page_key_offset(in_page, rank + i, hd), v);
+    }
+    const int tail = hd - rank;
+    for (int e = tid; e < n_heads * tail; e += blockDim.x) {
+        const int h = e / tail, i = e % tail;
+        float v = 0.f;
+        if (i < rot) {
+            const float* q = qfull + (size_t)t * ldq + (size_t)h * (dim + rot) + dim;
+            v = q[i];
+            if (i < rot_dims) {
+                const float2 c = tab[i >> 1];
+                const float other = q[i ^ 1];
+                v = (i & 1) ? fmaf(v, c.x, other * c.y) : fmaf(v, c.x, -other * c.y);
+            }
+        }
+        store_f32(q_out + ((size_t)t * n_heads + h) * hd + rank + i, v);
+    }
+}
+
+LLOGOS_EXPORT int llogos_latent_prepare(const float* kv, int ldkv, const float* qfull, int ldq, void* q_out, int dtype,
+                                        const float* norm_w, float eps, const void* cs, void* k_pool,
+                                        const int* table, int table_stride, const int* tok_seq, const int* tok_pos,
+                                        int T, int n_heads, int dim, int rot, int rot_dims, int rank, int hd,
+                                        hipStream_t stream) {
+    if (T <= 0 || n_heads <= 0 || dim < 0 || rot < 0 || rank <= 0 || hd < rank + rot || hd % 16) return LLOGOS_BAD_ARGUMENT;
+    if (rot_dims < 0 || rot_dims > rot || rot_dims % 2 || ldkv < rank + rot || ldq < n_heads * (dim + rot)) return LLOGOS_BAD_ARGUMENT;
+    PagedKV cache{table, table_stride, 1, hd};
+    if (dtype == DT_F32)
+        latent_prepare_kernel<float><<<T, 256, 0, stream>>>(kv, ldkv, qfull, ldq, (float*)q_out, norm_w, eps, (const float2*)cs,
+                                                            (float*)k_pool, cache, tok_seq, tok_pos, n_heads, dim, rot, rot_dims, rank, hd);
+    else if (dtype == DT_BF16)
+        latent_prepare_kernel<bf16_t><<<T, 256, 0, stream>>>(kv, ldkv, qfull, ldq, (bf16_t*)q_out, norm_w, eps, (const float2*)cs,
+                                                             (bf16_t*)k_pool, cache, tok_seq, tok_pos, n_heads, dim, rot, rot_dims, rank, hd);
+    else
+        return LLOGOS_BAD_ARGUMENT;
+    return LLOGOS_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------- one small product per head
+// out[t, h, n] = sum_k a[t, h, k] * w[h, n, k]   for n < N, k < K, every head with its own matrix.
+// a: row stride lda, head stride a_head; out: row stride ldo, head stride o_head; w [H, N, K] dense.
+// Tiles of 64 tokens x 64 outputs, 16 values of k at a time through LDS, 4 x 4 outputs a thread,
+// sums in 32-bit in ascending k: an output's sum does not depend on what else is in the step.
+template <typename TA, typename TW, typename TO>
+__global__ __launch_bounds__(256) void head_products_kernel(TO* __restrict__ out, int ldo, int o_head,
+                                                            const TA* __restrict__ a, int lda, int a_head,
+                                                            const TW* __restrict__ w, int M, int N, int K) {
+    __shared__ float sa[16][64 + 4];
+    __shared__ float sw[16][64 + 4];
+    const int h = blockIdx.z, m0 = blockIdx.x * 64, n0 = blockIdx.y * 64;
+    const int tid = threadIdx.x, tx = tid % 16, ty = tid / 16;
+    const TA* ah = a + (size_t)h * a_head;
+    const TW* wh = w + (size_t)h * N * K;
+    float acc[4][4] = {};
+    for (int k0 = 0; k0 < K; k0 += 16) {
+        for (int e = tid; e < 64 * 16; e += 256) {
+            const int r = e / 16, kk = e % 16;
+            sa[kk][r] = (m0 + r < M && k0 + kk < K) ? load_f32(ah + (size_t)(m0 + r) * lda + k0 + kk) : 0.f;
+            sw[kk][r] = (n0 + r < N && k0 + kk < K) ? load_f32(wh + (size_t)(n0 + r) * K + k0 + kk) : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < 16; ++kk) {
+            float av[4], wv[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { av[i] = sa[kk][ty * 4 + i]; wv[i] = sw[kk][tx * 4 + i]; }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int jn = 0; jn < 4; ++jn) acc[i][jn] = fmaf(av[i], wv[jn], acc[i][jn]);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int m = m0 + ty * 4 + i;
+        if (m >= M) continue;
+#pragma unroll
+        for (int jn = 0; jn < 4; ++jn) {
+            const int n = n0 + tx * 4 + jn;
+            if (n < N) store_f32(out + (size_t)m * ldo + (size_t)h * o_head + n, acc[i][jn]);
+        }
+    }
+}
+
+LLOGOS_EXPORT int llogos_head_products(void* out, int out_dtype, int ldo, int o_head, const void* a, int a_dtype, int lda,
+                                       int a_head, const void* w, int w_dtype, int M, int H, int N, int K, hipStream_t stream) {
+    if (M <= 0 || H <= 0 || N <= 0 || K <= 0) return LLOGOS_BAD_ARGUMENT;
+    dim3 grid((M + 63) / 64, (N + 63) / 64, H);
+#define HP(TA, TW, TO) head_products_kernel<TA, TW, TO><<<grid, 256, 0, stream>>>((TO*)out, ldo, o_head, (const TA*)a, lda, a_head, \
+        (const TW*)w, M, N, K)
+    if (a_dtype == DT_F32 && w_dtype == DT_F32 && out_dtype == DT_F32) HP(float, float, float);
+    else if (a_dtype == DT_F32 && w_dtype == DT_BF16 && out_dtype == DT_BF16) HP(float, bf16_t, bf16_t);
+    else if (a_dtype == DT_BF16 && w_dtype == DT_BF16 && out_dtype == DT_BF16) HP(bf16_t, bf16_t, bf16_t);
+    else if (a_dtype == DT_BF16 && w_dtype == DT_BF16 && out_dtype == DT_F32) HP(bf16_t, bf16_t, float);
+    else return LLOGOS_BAD_ARGUMENT;
+#undef HP
+    return LLOGOS_LAUNCH_CHECK();
+}

@@ -1,0 +1,292 @@
+// Kernels for parts that keep a fixed-size state for each sequence: a short causal
+// convolution over time, the mix of a token with the one before it, and a linear recurrence
+// with a matrix state per head.  State rows are indexed by cache slot (slots[seq]); a row
+// is zero when its slot is handed out.  All arithmetic is 32-bit; inputs and outputs may be
+// stored as float or bfloat16.
+#include "common.h"
+
+// ---------------------------------------------------------------- short causal convolution
+// out[t, c] = h[t, c] + sum_j w[c, j] * h_(t - taps + 1 + j)[c]   (w[c, taps - 1] multiplies token t)
+// Rows before the step's first token of a sequence come from the sequence's state
+// [taps - 1, W], whose row i holds the input at position (length - (taps - 1) + i); positions
+// before 0 count as zero.  cu (token offset of each sequence in the step) may be null: then
+// every sequence brings one token, and the thread that computes a channel also shifts the
+// channel's state (update_state).  For longer steps conv_state_kernel runs afterwards.
+constexpr int kMaxTaps = 16;
+
+template <typename TO>
+__global__ void causal_conv_kernel(TO* __restrict__ out, const float* __restrict__ h, const float* __restrict__ w,
+                                   float* __restrict__ state, const int* __restrict__ slots,
+                                   const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
+                                   const int* __restrict__ cu, int W, int taps, int update_state) {
+    const int t = blockIdx.x;
+    const int seq = tok_seq[t], pos = tok_pos[t];
+    const int before = cu ? t - cu[seq] : 0;                 // tokens of this sequence earlier in the step
+    float* st = state + (size_t)slots[seq] * (taps - 1) * W;
+    for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < W; c += gridDim.y * blockDim.x) {
+        const float* wc = w + (size_t)c * taps;
+        const float x0 = h[(size_t)t * W + c];
+        float acc = x0 * wc[taps - 1];
+        float old[kMaxTaps];
+#pragma unroll
+        for (int j = 1; j < kMaxTaps; ++j) {
+            if (j < taps) {
+                float v = 0.f;
+                if (j <= before) v = h[(size_t)(t - j) * W + c];
+                else if (pos - j >= 0) v = st[(size_t)(taps - 1 + before - j) * W + c];
+                old[j] = v;
+                acc = fmaf(wc[taps - 1 - j], v, acc);
+            }
+        }
+        store_f32(out + (size_t)t * W + c, x0 + acc);
+        if (update_state) {                                  // one token a sequence: row i <- row i + 1, last <- this token
+#pragma unroll
+            for (int j = 1; j < kMaxTaps; ++j)
+                if (j < taps) st[(size_t)(taps - 1 - j) * W + c] = (j == 1) ? x0 : old[j - 1];
+        }
+    }
+}
+
+// The state after a step of any length: row i <- the input at position new_len - (taps - 1) + i,
+// from this step's rows or from the old state.  A thread owns a channel of a sequence and
+// reads all it needs before it writes.
+__global__ void conv_state_kernel(const float* __restrict__ h, float* __restrict__ state, const int* __restrict__ slots,
+                                  const int* __restrict__ cu, int W, int taps) {
+    const int seq = blockIdx.x;
+    const int first = cu[seq], count = cu[seq + 1] - first;
+    float* st = state + (size_t)slots[seq] * (taps - 1) * W;
+    for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < W; c += gridDim.y * blockDim.x) {
+        float keep[kMaxTaps];
+#pragma unroll
+        for (int i = 0; i < kMaxTaps - 1; ++i) {
+            if (i < taps - 1) {
+                const int back = taps - 1 - i;               // this row is the input `back` tokens before the new end
+                keep[i] = back <= count ? h[(size_t)(first + count - back) * W + c] : st[(size_t)(i + count) * W + c];
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < kMaxTaps - 1; ++i)
+            if (i < taps - 1) st[(size_t)i * W + c] = keep[i];
+    }
+}
+
+LLOGOS_EXPORT int llogos_causal_conv(void* out, int out_dtype, const float* h, const float* w, float* state,
+                                     const int* slots, const int* tok_seq, const int* tok_pos, const int* cu,
+                                     int T, int B, int W, int taps, hipStream_t stream) {
+    if (T <= 0 || B <= 0 || W <= 0 || taps < 1 || taps > kMaxTaps) return LLOGOS_BAD_ARGUMENT;
+    if (!cu && T != B) return LLOGOS_BAD_ARGUMENT;
+    const int threads = 256;
+    const int by = (W + threads - 1) / threads;
+    dim3 grid(T, by);
+    const int fused = cu ? 0 : 1;
+    if (out_dtype == DT_F32)
+        causal_conv_kernel<float><<<grid, threads, 0, stream>>>((float*)out, h, w, state, slots, tok_seq, tok_pos, cu, W, taps, fused);
+    else if (out_dtype == DT_BF16)
+        causal_conv_kernel<bf16_t><<<grid, threads, 0, stream>>>((bf16_t*)out, h, w, state, slots, tok_seq, tok_pos, cu, W, taps, fused);
+    else
+        return LLOGOS_BAD_ARGUMENT;
+    if (cu && taps > 1) conv_state_kernel<<<dim3(B, by), threads, 0, stream>>>(h, state, slots, cu, W, taps);
+    return LLOGOS_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------- mix with the token before
+// out[s][t, c] = h[t, c] + (h_prev[c] - h[t, c]) * mu[s][c] for s < n_mix, where h_prev is the
+// row before in the step, or, for a sequence's first row of the step, the sequence's state row
+// `prev` (zero at the start of a sequence).  The state is not written here: the recurrence
+// kernel, which runs after every reader, stores the step's last row.
+template <typename TO>
+__global__ void token_shift_kernel(TO* __restrict__ out, const float* __restrict__ h, const float* __restrict__ mu,
+                                   const float* __restrict__ state, size_t state_stride, const int* __restrict__ slots,
+                                   const int* __restrict__ tok_seq, const int* __restrict__ cu, int T, int W, int n_mix) {
+    const int t = blockIdx.x;
+    const int seq = tok_seq[t];
+    const bool first = cu ? (t == cu[seq]) : true;
+    const float* prev = first ? state + (size_t)slots[seq] * state_stride : h + (size_t)(t - 1) * W;
+    for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < W; c += gridDim.y * blockDim.x) {
+        const float x = h[(size_t)t * W + c];
+        const float d = prev[c] - x;
+        for (int s = 0; s < n_mix; ++s)
+            store_f32(out + ((size_t)s * T + t) * W + c, fmaf(d, mu[(size_t)s * W + c], x));
+    }
+}
+
+LLOGOS_EXPORT int llogos_token_shift(void* out, int out_dtype, const float* h, const float* mu, const float* state,
+                                     long long state_stride, const int* slots, const int* tok_seq, const int* cu,
+                                     int T, int W, int n_mix, hipStream_t stream) {
+    if (T <= 0 || W <= 0 || n_mix <= 0) return LLOGOS_BAD_ARGUMENT;
+    const int threads = 256;
+    dim3 grid(T, (W + threads - 1) / threads);
+    if (out_dtype == DT_F32)
+        token_shift_kernel<float><<<grid, threads, 0, stream>>>((float*)out, h, mu, state, (size_t)state_stride, slots, tok_seq, cu, T, W, n_mix);
+    else if (out_dtype == DT_BF16)
+        token_shift_kernel<bf16_t><<<grid, threads, 0, stream>>>((bf16_t*)out, h, mu, state, (size_t)state_stride, slots, tok_seq, cu, T, W, n_mix);
+    else
+        return LLOGOS_BAD_ARGUMENT;
+    return LLOGOS_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------- recurrence with a matrix state per head
+// Per sequence and head, with S [key channel i, value channel j] carried from token to token:
+//     o_t[j] = sum_i r_t[i] * (S[i, j] + u[i] * k_t[i] * v_t[j])
+//     S[i, j] <- w_t[i] * S[i, j] + k_t[i] * v_t[j],      w_t[i] = exp(-exp(d_t[i] + w0[i]))
+// then y_t = o_t / sqrt(mean_j(o_t^2) + eps) * g[j] * silu(gate_t[j]) over the head's D channels.
+// r, k, v, d, gate are float [T, H * D] (row stride ld); y is [T, H * D] in the output type.
+//
+// One block per (sequence, head).  Thread (j, part) keeps rows [part * rpt, (part + 1) * rpt) of
+// column j of S in registers; the P parts of a column are neighbouring lanes and add their
+// sums by shuffles, so the token loop needs no barrier.  Tokens go through LDS in chunks: a
+// chunk's r, k, w, v are loaded by all threads, its outputs are normed and stored by all
+// threads after the chunk's loop.  The state is stored [H][j][i] (a thread's rows in a row).
+// After its last token the block with head 0 copies the step's last mixer input row to the
+// sequence's `prev` state (the token-shift kernel has read the old one by then).
+constexpr int kScanChunk = 16;
+
+template <int RPT, typename TO>
+__global__ void wkv_scan_kernel(TO* __restrict__ y, const float* __restrict__ r, const float* __restrict__ k,
+                                const float* __restrict__ v, const float* __restrict__ d, const float* __restrict__ gate,
+                                int ld, const float* __restrict__ w0, const float* __restrict__ u,
+                                const float* __restrict__ g, float eps,
+                                float* __restrict__ state, size_t state_stride, size_t prev_offset,
+                                const float* __restrict__ h_in, int W,
+                                const int* __restrict__ slots, const int* __restrict__ cu,
+                                int H, int D, int P, int rpt) {
+    extern __shared__ float smem[];
+    const int seq = blockIdx.x, head = blockIdx.y;
+    const int first = cu ? cu[seq] : seq, count = cu ? cu[seq + 1] - first : 1;
+    const int tid = threadIdx.x, nthreads = blockDim.x;
+    const int j = tid / P, part = tid % P;
+    const bool active = j < D;
+    const int i0 = part * rpt;
+    float* s_r = smem;                          // [chunk][D]
+    float* s_k = s_r + kScanChunk * D;
+    float* s_w = s_k + kScanChunk * D;
+    float* s_v = s_w + kScanChunk * D;
+    float* s_o = s_v + kScanChunk * D;
+    float* s_u = s_o + kScanChunk * D;          // [D]
+    float* row = state + (size_t)slots[seq] * state_stride;
+    float* S = row + ((size_t)head * D + (active ? j : 0)) * D + i0;
+
+    float s[RPT];
+#pragma unroll
+    for (int m = 0; m < RPT; ++m) s[m] = (active && m < rpt && i0 + m < D) ? S[m] : 0.f;
+    for (int i = tid; i < D; i += nthreads) s_u[i] = u[head * D + i];
+
+    const size_t col0 = (size_t)head * D;
+    for (int c0 = 0; c0 < count; c0 += kScanChunk) {
+        const int n = min(kScanChunk, count - c0);
+        __syncthreads();                        // the chunk before has been normed and stored
+        for (int e = tid; e < n * D; e += nthreads) {
+            const int c = e / D, i = e % D;
+            const size_t at = (size_t)(first + c0 + c) * ld + col0 + i;
+            s_r[e] = r[at];
+            s_k[e] = k[at];
+            s_v[e] = v[at];
+            s_w[e] = expf(-expf(d[at] + w0[col0 + i]));
+        }
+        __syncthreads();
+        for (int c = 0; c < n; ++c) {
+            const float* rr = s_r + c * D + i0;
+            const float* kk = s_k + c * D + i0;
+            const float* ww = s_w + c * D + i0;
+            const float vj = active ? s_v[c * D + j] : 0.f;
+            float acc = 0.f;
+#pragma unroll
+            for (int m = 0; m < RPT; ++m) {
+                if (m < rpt && i0 + m < D) {
+                    const float kv = kk[m] * vj;
+                    acc = fmaf(rr[m], fmaf(s_u[i0 + m], kv, s[m]), acc);
+                    s[m] = fmaf(ww[m], s[m], kv);
+                }
+            }
+            for (int o = 1; o < P; o <<= 1) acc += __shfl_xor(acc, o, kWave);
+            if (active && part == 0) s_o[c * D + j] = acc;
+        }
+        __syncthreads();
+        // norm over the head, weight, gate: a wave takes a token at a time
+        const int wave = tid / kWave, lane = tid % kWave, nwaves = (nthreads + kWave - 1) / kWave;
+        for (int c = wave; c < n; c += nwaves) {
+            float ss = 0.f;
+            for (int i = lane; i < D; i += kWave) { const float o = s_o[c * D + i]; ss = fmaf(o, o, ss); }
+            ss = wave_sum(ss);
+            const float inv = 1.0f / sqrtf(ss / (float)D + eps);
+            const size_t base = (size_t)(first + c0 + c);
+            for (int i = lane; i < D; i += kWave) {
+                const float z = gate[base * ld + col0 + i];
+                const float sg = z / (1.0f + expf(-z));
+                store_f32(y + base * (size_t)H * D + col0 + i, s_o[c * D + i] * inv * g[col0 + i] * sg);
+            }
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < RPT; ++m)
+        if (active && m < rpt && i0 + m < D) S[m] = s[m];
+    if (head == 0 && h_in) {
+        const float* last = h_in + (size_t)(first + count - 1) * W;
+        for (int c = tid; c < W; c += nthreads) row[prev_offset + c] = last[c];
+    }
+}
+
+LLOGOS_EXPORT int llogos_wkv_scan(void* y, int out_dtype, const float* r, const float* k, const float* v, const float* d,
+                                  const float* gate, int ld, const float* w0, const float* u, const float* g, float eps,
+                                  float* state, long long state_stride, long long prev_offset, const float* h_in, int W,
+                                  const int* slots, const int* cu, int B, int H, int D, hipStream_t stream) {
+    if (B <= 0 || H <= 0 || D <= 0 || ld < H * D) return LLOGOS_BAD_ARGUMENT;
+    if (D > 256) return LLOGOS_UNSUPPORTED;
+    // parts of a column: a power of two, rows a part <= 16 where the block then stays within 1024 threads
+    int rpt_max = 16, P = 1;
+    while (P * rpt_max < D) P <<= 1;
+    if ((long long)D * P > 1024) { rpt_max = 64; P = 1; while (P * rpt_max < D) P <<= 1; }
+    const int rpt = (D + P - 1) / P;
+    int threads = D * P;
+    threads = (threads + kWave - 1) / kWave * kWave;
+    if (threads > 1024) return LLOGOS_UNSUPPORTED;
+    const size_t smem = (size_t)(5 * kScanChunk + 1) * D * sizeof(float);
+    dim3 grid(B, H);
+#define SCAN(RPT, TO) wkv_scan_kernel<RPT, TO><<<grid, threads, smem, stream>>>((TO*)y, r, k, v, d, gate, ld, w0, u, g, eps, \
+        state, (size_t)state_stride, (size_t)prev_offset, h_in, W, slots, cu, H, D, P, rpt)
+    if (out_dtype == DT_F32) { if (rpt_max == 16) SCAN(16, float); else SCAN(64, float); }
+    else if (out_dtype == DT_BF16) { if (rpt_max == 16) SCAN(16, bf16_t); else SCAN(64, bf16_t); }
+    else return LLOGOS_BAD_ARGUMENT;
+#undef SCAN
+    return LLOGOS_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------- activations of a product
+// out = act(sum of the parts of `in`) element by element.  kinds:
+//   0 tanh;  1 silu;  2 gelu (tanh form);
+//   3 the piecewise xIELU with a = softplus(p), b = 1/2 + softplus(q):
+//       z > 0: a z^2 + z / 2;   z <= 0: b (exp(z) - 1 - z) + z / 2
+enum { ACT_TANH = 0, ACT_SILU = 1, ACT_GELU_TANH = 2, ACT_XIELU = 3 };
+
+__device__ __forceinline__ float activate(float z, int kind, float a, float b) {
+    switch (kind) {
+        case ACT_TANH: return tanhf(z);
+        case ACT_SILU: return z / (1.0f + expf(-z));
+        case ACT_GELU_TANH: return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+        default: return z > 0.f ? fmaf(a * z, z, 0.5f * z) : fmaf(b, expm1f(z) - z, 0.5f * z);
+    }
+}
+
+template <typename TO, typename TI>
+__global__ void activation_kernel(TO* __restrict__ out, const TI* __restrict__ in, int parts, size_t part_stride,
+                                  size_t n, int kind, float a, float b) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    float z = load_f32(in + i);
+    for (int q = 1; q < parts; ++q) z += load_f32(in + q * part_stride + i);
+    store_f32(out + i, activate(z, kind, a, b));
+}
+
+LLOGOS_EXPORT int llogos_activation(void* out, int out_dtype, const void* in, int in_dtype, int parts, long long part_stride,
+                                    long long n, int kind, float a, float b, hipStream_t stream) {
+    if (n <= 0 || parts < 1 || kind < 0 || kind > ACT_XIELU) return LLOGOS_BAD_ARGUMENT;
+    const unsigned blocks = (unsigned)((n + 255) / 256);
+#define ACT(TO, TI) activation_kernel<TO, TI><<<blocks, 256, 0, stream>>>((TO*)out, (const TI*)in, parts, (size_t)part_stride, (size_t)n, kind, a, b)
+    if (out_dtype == DT_F32 && in_dtype == DT_F32) ACT(float, float);
+    else if (out_dtype == DT_BF16 && in_dtype == DT_F32) ACT(bf16_t, float);
+    else if (out_dtype == DT_BF16 && in_dtype == DT_BF16) ACT(bf16_t, bf16_t);
+    else if (out_dtype == DT_F32 && in_dtype == DT_BF16) ACT(float, bf16_t);
+    else return LLOGOS_BAD_ARGUMENT;
+#undef ACT
+    return LLOGOS_LAUNCH_CHECK();
+}

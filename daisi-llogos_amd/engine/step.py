@@ -65,7 +65,7 @@ def packed_weight_budget(model: Model, dtype: torch.dtype, max_tokens: int, devi
             for d in spec.shape:
                 n *= int(d)
             elements += n
-    cache = max_tokens * sum(2 * kv.n_kv_heads * kv.head_dim * element for kv, _ in model.cache_needs() if kv is not None)
+    cache = max_tokens * sum((2 if kv.values else 1) * kv.n_kv_heads * kv.head_dim * element for kv, _ in model.cache_needs() if kv is not None)
     with torch.cuda.device(device):
         free, total = torch.cuda.mem_get_info()
         free += torch.cuda.memory_reserved() - torch.cuda.memory_allocated()      # what torch holds but does not use
@@ -121,10 +121,10 @@ class Engine:
         dev = require_gpu(device)
         data = read_config_json(folder)
         arch = architecture_of(data)
-        config = arch.read_config(data)
-        model = Model(arch.model_spec(config, **spec_options))
         ckpt = Checkpoint(folder)
         try:
+            config = arch.read_config(data, shapes=ckpt.shapes()) if arch.reads_shapes else arch.read_config(data)
+            model = Model(arch.model_spec(config, **spec_options))
             tied = model.spec.head_name + ".weight" if model.spec.tie_head else None
             ckpt.check(model.tensor_specs(), tied_head=tied)
             rt = Runtime(dev, resolve_dtype(dtype))

@@ -8,7 +8,7 @@ from typing import Callable, Dict, List, Optional, Tuple
 import torch
 
 from ..ops import kernels as K
-from ..parts.base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, KVSpec, LayerCache, Mixer, Part, Runtime, StateSpec,
+from ..parts.base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, OTHER_PARTS, KVSpec, LayerCache, Mixer, Part, Runtime, StateSpec,
                           StepContext, TensorSpec, make)
 from ..parts.linear import Linear, _to_device
 
@@ -18,7 +18,7 @@ class LayerSpec:
     """Kinds and parameters of one layer's parts.  The four named fields are the parts of the
     pre-norm block; a block of another arrangement (two mixers side by side, a mixer alone)
     names its parts in `more`: keyword of the block's constructor -> (registry, kind,
-    parameters) with registry one of 'mixer', 'feed_forward', 'norm', or a list of such triples."""
+    parameters) with registry one of 'mixer', 'feed_forward', 'norm', 'part', or a list of such triples."""
     mixer: Optional[Tuple[str, dict]] = None
     ffn: Optional[Tuple[str, dict]] = None
     mixer_norm: Optional[Tuple[str, dict]] = None
@@ -53,7 +53,8 @@ class ModelSpec:
     logit_softcap: float = 0.0     # ... and then, if > 0, bent to cap * tanh(logit / cap)
 
 
-_REGISTRIES = {"mixer": (MIXERS, "mixer"), "feed_forward": (FEED_FORWARDS, "feed-forward"), "norm": (NORMS, "norm")}
+_REGISTRIES = {"mixer": (MIXERS, "mixer"), "feed_forward": (FEED_FORWARDS, "feed-forward"), "norm": (NORMS, "norm"),
+               "part": (OTHER_PARTS, "part")}
 
 
 def _make_part(triple):
@@ -78,8 +79,8 @@ def build_layer(spec: LayerSpec):
 class Model:
     """Built from a ModelSpec; bound to device tensors by `bind`; `forward` runs one step.
 
-    The cache is asked for by *unit*: one unit for each mixer of each scheduled run, in the
-    order of the schedule and, within a run, of the block's mixers()."""
+    The cache is asked for by *unit*: one unit for each mixer (and each other part with state) of
+    each scheduled run, in the order of the schedule and, within a run, of the block's cache_parts()."""
 
     def __init__(self, spec: ModelSpec):
         self.spec = spec
@@ -92,7 +93,7 @@ class Model:
         for e in self.schedule:
             if not 0 <= e.layer < len(self.layers):
                 raise ValueError(f"a schedule entry names layer {e.layer}, the model has {len(self.layers)}")
-            mixers = self.layers[e.layer].mixers()
+            mixers = self.layers[e.layer].cache_parts()       # the mixers, and whatever else keeps state
             self.entry_units.append(list(range(len(self.unit_mixers), len(self.unit_mixers) + len(mixers))))
             self.unit_mixers += mixers
         self._check_schedule()
@@ -108,8 +109,8 @@ class Model:
                 src = self.schedule[e.cache_of]
                 if src.cache_of is not None:
                     raise ValueError(f"schedule entry {i} must read from an entry that owns its cache")
-                mine = [m.kv_spec() for m in self.layers[e.layer].mixers()]
-                theirs = [m.kv_spec() for m in self.layers[src.layer].mixers()]
+                mine = [m.kv_spec() for m in self.layers[e.layer].cache_parts()]
+                theirs = [m.kv_spec() for m in self.layers[src.layer].cache_parts()]
                 if mine != theirs:
                     raise ValueError(f"schedule entry {i} and entry {e.cache_of} need different key/value storage")
 

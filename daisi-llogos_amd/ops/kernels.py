@@ -88,10 +88,13 @@ def _parts(t: Optional[torch.Tensor]) -> Tuple[int, int]:
     return t.shape[0], t.stride(0)
 
 
-def _check_pools(k_pool: torch.Tensor, v_pool: torch.Tensor, n_kv_heads: int, head_dim: int, who: str) -> None:
+def _check_pools(k_pool: torch.Tensor, v_pool: Optional[torch.Tensor], n_kv_heads: int, head_dim: int, who: str) -> None:
     _need(head_dim % 16 == 0, f"{who}: head size {head_dim} is not a multiple of 16")
     _need(tuple(k_pool.shape[1:]) == (n_kv_heads, PAGE_TOKENS * head_dim),
           f"{who}: key pool must be [pages, kv_heads, {PAGE_TOKENS} * head_dim]")
+    if v_pool is None:          # a cache whose values are part of its key rows
+        _need(k_pool.is_contiguous(), f"{who}: the pool must be contiguous")
+        return
     _need(tuple(v_pool.shape) == tuple(k_pool.shape),
           f"{who}: value pool must be [pages, kv_heads, {PAGE_TOKENS} * head_dim] like the key pool")
     _need(k_pool.is_contiguous() and v_pool.is_contiguous(), f"{who}: the pools must be contiguous")
@@ -181,14 +184,14 @@ def gemm_generic(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor],
     return out
 
 
-def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor) -> torch.Tensor:
-    """[T, half, 2] float32 (cos, sin) of positions[t] * inv_freq[i], computed in double."""
+def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, amplitude: float = 1.0) -> torch.Tensor:
+    """[T, half, 2] float32 (cos, sin) of positions[t] * inv_freq[i], computed in double, times `amplitude`."""
     _dev(positions, inv_freq)
     _i32(positions, "positions")
     _need(inv_freq.dtype == torch.float64 and inv_freq.dim() == 1, "rope_table: inv_freq must be float64 [half]")
     T, half = positions.numel(), inv_freq.numel()
     cs = torch.empty((T, half, 2), dtype=torch.float32, device=positions.device)
-    _check(_lib().llogos_rope_table(_p(cs), _p(positions), _p(inv_freq), T, half, _stream()), "rope_table")
+    _check(_lib().llogos_rope_table(_p(cs), _p(positions), _p(inv_freq), T, half, ctypes.c_double(amplitude), _stream()), "rope_table")
     return cs
 
 
@@ -234,9 +237,12 @@ def qk_rope_cache(qkv: torch.Tensor, bias: Optional[torch.Tensor], out_dtype: to
 def attention_generic(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torch.Tensor,
                       table: torch.Tensor, tok_seq: torch.Tensor, tok_pos: torch.Tensor,
                       n_heads: int, n_kv_heads: int, head_dim: int, scale: float,
-                      window: int = 0, sinks: int = 0) -> torch.Tensor:
+                      window: int = 0, sinks: int = 0, v_dim: Optional[int] = None,
+                      head_sink: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention of T query rows (row stride `q_stride` elements, heads first) over the
-    paged cache; returns [T, n_heads * head_dim] in the cache's element type."""
+    paged cache; returns [T, n_heads * v_dim] in the cache's element type.  `v_pool` None:
+    a value is the first `v_dim` dimensions of its key row.  `head_sink` float32 [n_heads]:
+    a learned score per head that joins the softmax's denominator without a key or a value."""
     _dev(k_pool, v_pool, table, tok_seq, tok_pos)
     _i32(tok_seq, "tok_seq"); _i32(tok_pos, "tok_pos"); _i32(table, "table")
     T = tok_seq.numel()
@@ -246,11 +252,16 @@ def attention_generic(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_po
     _check_pools(k_pool, v_pool, n_kv_heads, head_dim, "attention")
     _need(q_stride >= n_heads * head_dim and q.numel() >= (T - 1) * q_stride + n_heads * head_dim,
           "attention: q too small")
-    out = torch.empty((T, n_heads * head_dim), dtype=q.dtype, device=q.device)
+    v_dim = head_dim if v_dim is None else int(v_dim)
+    _need(0 < v_dim <= head_dim, "attention: value width outside 1..head_dim")
+    if head_sink is not None:
+        _dev(head_sink)
+        _need(head_sink.dtype == torch.float32 and head_sink.shape == (n_heads,), "attention: head_sink must be float32 [n_heads]")
+    out = torch.empty((T, n_heads * v_dim), dtype=q.dtype, device=q.device)
     _check(_lib().llogos_attention_generic(
         _p(out), _p(q), _dt(q), q_stride, _p(k_pool), _p(v_pool), _p(table), table.stride(0),
         _p(tok_seq), _p(tok_pos), T, n_heads, n_kv_heads, head_dim, ctypes.c_float(scale),
-        window, sinks, _stream()), "attention_generic")
+        window, sinks, v_dim, _p(head_sink), _stream()), "attention_generic")
     return out
 
 
@@ -289,6 +300,137 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
     R, V = logits.shape
     out = torch.empty((R,), dtype=torch.int32, device=logits.device)
     _check(_lib().llogos_argmax(_p(out), _p(logits), R, V, _stream()), "argmax")
+    return out
+
+
+# ----------------------------------------------------------------------------
+# parts with a fixed-size state per sequence
+# ----------------------------------------------------------------------------
+MAX_CONV_TAPS = 16
+ACTIVATIONS = {"tanh": 0, "silu": 1, "gelu_tanh": 2, "xielu": 3}
+
+
+def causal_conv(ctx, h: torch.Tensor, w: torch.Tensor, state: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """h + conv(h) over time, channel by channel: h float32 [T, W] (the step's rows, one sequence
+    after the other), w float32 [W, taps] whose last tap multiplies the present token, state
+    float32 [slots, taps - 1, W]: a sequence's last taps - 1 inputs, read for the rows before the
+    step's first and brought up to date."""
+    _dev(h, w, state, ctx.slots, ctx.tok_seq, ctx.tok_pos, ctx.cu_dev)
+    _need(h.dtype == torch.float32 and h.dim() == 2, "causal_conv: h must be float32 [T, W]")
+    T, W = h.shape
+    _need(w.dtype == torch.float32 and w.dim() == 2 and w.shape[0] == W and 1 <= w.shape[1] <= MAX_CONV_TAPS,
+          f"causal_conv: w must be float32 [W, taps] with at most {MAX_CONV_TAPS} taps")
+    taps = w.shape[1]
+    _need(state.dtype == torch.float32 and state.dim() == 3 and tuple(state.shape[1:]) == (max(taps - 1, 0), W),
+          "causal_conv: state must be float32 [slots, taps - 1, W]")
+    _need(T == ctx.n_tokens and ctx.tok_seq.numel() == T and ctx.tok_pos.numel() == T, "causal_conv: one row a token of the step")
+    _need(ctx.cu_dev is not None or T == ctx.batch, "causal_conv: a step of several tokens a sequence needs the token offsets")
+    out = torch.empty((T, W), dtype=out_dtype, device=h.device)
+    _check(_lib().llogos_causal_conv(_p(out), _DT[out_dtype], _p(h), _p(w), _p(state), _p(ctx.slots), _p(ctx.tok_seq),
+                                     _p(ctx.tok_pos), _p(ctx.cu_dev), T, ctx.batch, W, taps, _stream()), "causal_conv")
+    return out
+
+
+def token_shift(ctx, h: torch.Tensor, mu: torch.Tensor, prev: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """[n, T, W]: h + (row before - h) * mu[s] for each of the n rows of mu; the row before a
+    sequence's first row of the step is prev[slot] (`prev` float32 [slots, W], maybe a column
+    range of a wider state tensor; it is read, not written)."""
+    _dev(h, mu, ctx.slots, ctx.tok_seq, ctx.cu_dev)
+    _need(h.dtype == torch.float32 and h.dim() == 2, "token_shift: h must be float32 [T, W]")
+    T, W = h.shape
+    _need(mu.dtype == torch.float32 and mu.dim() == 2 and mu.shape[1] == W, "token_shift: mu must be float32 [n, W]")
+    _need(prev.is_cuda and prev.dtype == torch.float32 and prev.dim() == 2 and prev.shape[1] == W and prev.stride(1) == 1,
+          "token_shift: prev must be float32 [slots, W]")
+    _need(ctx.cu_dev is not None or T == ctx.batch, "token_shift: a step of several tokens a sequence needs the token offsets")
+    n = mu.shape[0]
+    out = torch.empty((n, T, W), dtype=out_dtype, device=h.device)
+    _check(_lib().llogos_token_shift(_p(out), _DT[out_dtype], _p(h), _p(mu), _p(prev), ctypes.c_longlong(prev.stride(0)),
+                                     _p(ctx.slots), _p(ctx.tok_seq), _p(ctx.cu_dev), T, W, n, _stream()), "token_shift")
+    return out
+
+
+def wkv_scan(ctx, r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, d: torch.Tensor, gate: torch.Tensor,
+             w0: torch.Tensor, u: torch.Tensor, g: torch.Tensor, eps: float, state: torch.Tensor, n_heads: int,
+             dim: int, h_in: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """The recurrence S <- diag(w) S + k v^T with output (S + diag(u) k v^T)^T r per head, the
+    per-head RMS scale, weight g and silu(gate), over the step's rows of each sequence in turn.
+    r, k, v, d, gate: float32 [T, heads * dim] (w = exp(-exp(d + w0))); state float32
+    [slots, heads * dim * dim + W]: each head's S as [value channel][key channel], then the
+    last mixer input row, which this kernel replaces by h_in's last row of each sequence."""
+    HD = n_heads * dim
+    _dev(r, k, v, d, gate, w0, u, g, state, h_in, ctx.slots, ctx.cu_dev)
+    for t, name in ((r, "r"), (k, "k"), (v, "v"), (d, "d"), (gate, "gate")):
+        _need(t.dtype == torch.float32 and t.dim() == 2 and t.shape == (ctx.n_tokens, HD), f"wkv_scan: {name} must be float32 [T, heads * dim]")
+    for t, name in ((w0, "w0"), (u, "u"), (g, "g")):
+        _need(t.dtype == torch.float32 and t.numel() == HD, f"wkv_scan: {name} must be float32 [heads * dim]")
+    W = h_in.shape[1]
+    _need(h_in.dtype == torch.float32 and h_in.shape == (ctx.n_tokens, W), "wkv_scan: h_in must be float32 [T, W]")
+    _need(state.dtype == torch.float32 and state.dim() == 2 and state.shape[1] == HD * dim + W, "wkv_scan: state must be float32 [slots, heads * dim * dim + W]")
+    _need(ctx.cu_dev is not None or ctx.n_tokens == ctx.batch, "wkv_scan: a step of several tokens a sequence needs the token offsets")
+    _need((5 * 16 + 1) * dim * 4 <= 65536, f"wkv_scan: head size {dim} is too large")
+    y = torch.empty((ctx.n_tokens, HD), dtype=out_dtype, device=r.device)
+    _check(_lib().llogos_wkv_scan(_p(y), _DT[out_dtype], _p(r), _p(k), _p(v), _p(d), _p(gate), HD, _p(w0), _p(u), _p(g),
+                                  ctypes.c_float(eps), _p(state), ctypes.c_longlong(state.stride(0)), ctypes.c_longlong(HD * dim),
+                                  _p(h_in), W, _p(ctx.slots), _p(ctx.cu_dev), ctx.batch, n_heads, dim, _stream()), "wkv_scan")
+    return y
+
+
+def activation(x: torch.Tensor, kind: str, out_dtype: torch.dtype, a: float = 0.0, b: float = 0.0) -> torch.Tensor:
+    """act(x) element by element; x [T, N] or float32 partial sums [parts, T, N] that are added first.
+    kinds: tanh, silu, gelu_tanh, xielu (z > 0: a z^2 + z / 2; z <= 0: b (exp(z) - 1 - z) + z / 2)."""
+    _dev(x)
+    _need(kind in ACTIVATIONS, f"activation: unknown kind '{kind}'; known: {sorted(ACTIVATIONS)}")
+    parts, part_stride = _parts(x)
+    _need(parts == 1 or x.dtype == torch.float32, "activation: parts must be float32")
+    T, N = x.shape[-2:]
+    out = torch.empty((T, N), dtype=out_dtype, device=x.device)
+    if out.numel():
+        _check(_lib().llogos_activation(_p(out), _DT[out_dtype], _p(x), _dt(x), parts, ctypes.c_longlong(part_stride),
+                                        ctypes.c_longlong(T * N), ACTIVATIONS[kind], ctypes.c_float(a), ctypes.c_float(b), _stream()),
+               "activation")
+    return out
+
+
+# ----------------------------------------------------------------------------
+# attention through a latent
+# ----------------------------------------------------------------------------
+def latent_prepare(ctx, kv: torch.Tensor, qfull: torch.Tensor, q_out: torch.Tensor, norm_w: torch.Tensor, eps: float,
+                   cs: Optional[torch.Tensor], k_pool: torch.Tensor, table: torch.Tensor, n_heads: int, dim: int, rot: int,
+                   rot_dims: int, rank: int) -> None:
+    """From kv float32 [T, rank + rot] and qfull float32 [T, heads * (dim + rot)]: the normed latent and
+    the rotated shared key part go to the token's key row in the cache ([rank | rot | zeros]); each
+    head's rotated query part goes to q_out[t, h, rank:] ([T, heads, hd], hd the cache's row width)."""
+    _dev(kv, qfull, q_out, norm_w, cs, k_pool, table, ctx.tok_seq, ctx.tok_pos)
+    _i32(table, "table")
+    T = ctx.n_tokens
+    hd = q_out.shape[-1]
+    _need(kv.dtype == torch.float32 and kv.shape == (T, rank + rot), "latent_prepare: kv must be float32 [T, rank + rot]")
+    _need(qfull.dtype == torch.float32 and qfull.shape == (T, n_heads * (dim + rot)), "latent_prepare: q must be float32 [T, heads * (dim + rot)]")
+    _need(q_out.shape == (T, n_heads, hd) and q_out.dtype == k_pool.dtype, "latent_prepare: q_out must be [T, heads, hd] of the cache's type")
+    _need(hd % 16 == 0 and hd >= rank + rot, "latent_prepare: the cache's row is too narrow")
+    _check_pools(k_pool, None, 1, hd, "latent_prepare")
+    _need(norm_w.dtype == torch.float32 and norm_w.shape == (rank,), "latent_prepare: norm weight must be float32 [rank]")
+    _need(rot_dims % 2 == 0 and 0 <= rot_dims <= rot, "latent_prepare: rotated dimensions must be even and within rot")
+    if rot_dims:
+        _need(cs is not None and cs.dtype == torch.float32 and cs.shape == (T, rot_dims // 2, 2), "latent_prepare: rotary table shape")
+    _need(table.dim() == 2, "latent_prepare: page table must be [batch, pages]")
+    _check(_lib().llogos_latent_prepare(_p(kv), kv.stride(0), _p(qfull), qfull.stride(0), _p(q_out), _dt(q_out), _p(norm_w),
+                                        ctypes.c_float(eps), _p(cs), _p(k_pool), _p(table), table.stride(0), _p(ctx.tok_seq),
+                                        _p(ctx.tok_pos), T, n_heads, dim, rot, rot_dims, rank, hd, _stream()), "latent_prepare")
+
+
+def head_products(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[t, h, :N] = w[h] . a[t, h, :K] for every head h: a [T, H, >= K] and out [T, H, >= N] may be
+    views with their own row and head strides; w [H, N, K] is dense."""
+    _need(a.is_cuda and w.is_cuda and out.is_cuda and w.is_contiguous(), "head_products: device tensors, dense w")
+    _need(a.dim() == 3 and out.dim() == 3 and w.dim() == 3, "head_products: a [T, H, K], w [H, N, K], out [T, H, N]")
+    T, H, K = a.shape
+    N = w.shape[1]
+    _need(w.shape == (H, N, K) and out.shape == (T, H, N), "head_products: shapes do not fit")
+    _need(a.stride(2) == 1 and out.stride(2) == 1, "head_products: unit inner strides")
+    if T:
+        _check(_lib().llogos_head_products(_p(out), _dt(out), out.stride(0), out.stride(1), _p(a), _dt(a), a.stride(0), a.stride(1),
+                                           _p(w), _dt(w), T, H, N, K, _stream()), "head_products")
     return out
 
 

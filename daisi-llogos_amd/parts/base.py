@@ -46,6 +46,7 @@ class KVSpec:
     head_dim: int
     window: int = 0
     sinks: int = 0
+    values: bool = True     # False: no value pool; the mixer's values are part of its key rows (a latent cache)
 
 
 @dataclass(frozen=True)
@@ -186,6 +187,9 @@ class Mixer(Part):
 
     takes_normed_rows = False
     adds_to_residual = False
+    # True: h is to come as float32 rows (a mixer that mixes or norms its input again before its
+    # first product); a block whose producer can write either type asks it for that one
+    takes_float32_rows = False
 
     def kv_spec(self) -> Optional[KVSpec]:
         return None
@@ -265,6 +269,12 @@ class Block(Part):
     def feed_forwards(self) -> List["FeedForward"]:
         return []
 
+    def cache_parts(self) -> List[Part]:
+        """The parts that keep something in the cache for each sequence, in the order in which
+        forward() takes their LayerCaches: the mixers, unless a block has other parts with state
+        (each such part has kv_spec() and state_spec() like a mixer)."""
+        return self.mixers()
+
     def parts(self) -> List[Part]:
         raise NotImplementedError
 
@@ -299,6 +309,7 @@ FEED_FORWARDS: Dict[str, type] = {}
 NORMS: Dict[str, type] = {}
 POSITIONS: Dict[str, type] = {}
 BLOCKS: Dict[str, type] = {}
+OTHER_PARTS: Dict[str, type] = {}      # parts that are none of the above (a convolution in front of a sublayer)
 
 
 def _register(table: Dict[str, type], what: str):
@@ -315,6 +326,7 @@ register_feed_forward = _register(FEED_FORWARDS, "feed-forward")
 register_norm = _register(NORMS, "norm")
 register_position = _register(POSITIONS, "position encoding")
 register_block = _register(BLOCKS, "block")
+register_part = _register(OTHER_PARTS, "part")
 
 
 def make(table: Dict[str, type], what: str, kind: str, **params):

@@ -59,3 +59,81 @@ class PreNormBlock(Block):
             d = self.ffn.forward(ctx, h)
         mark(ctx, "feed_forward")
         return x, d
+
+
+@register_block("sandwich")
+class SandwichBlock(Block):
+    """Norms before and after each sublayer, and optionally a short convolution over time on what a
+    sublayer reads:
+
+        x += post_mixer_norm(mixer(conv1(mixer_norm(x))));   x += post_ffn_norm(ffn(conv2(ffn_norm(x))))
+
+    The feed-forward (with its norms and convolution) may be absent.  The normed outputs are float32
+    deltas: the first is added by the kernel of the norm that follows, the second is handed on as
+    `pending`.  The convolutions keep state for each sequence, so they are cache parts of the block
+    beside its mixer."""
+
+    def __init__(self, mixer_norm: Norm, mixer: Mixer, post_mixer_norm: Norm, ffn_norm: Optional[Norm] = None,
+                 ffn: Optional[FeedForward] = None, post_ffn_norm: Optional[Norm] = None,
+                 mixer_conv: Optional[Part] = None, ffn_conv: Optional[Part] = None):
+        if (ffn is None) != (ffn_norm is None) or (ffn is None) != (post_ffn_norm is None):
+            raise ValueError("a feed-forward comes with a norm before and a norm after it, or not at all")
+        if ffn is None and ffn_conv is not None:
+            raise ValueError("a convolution in front of a feed-forward that is not there")
+        self.mixer_norm, self.mixer, self.post_mixer_norm = mixer_norm, mixer, post_mixer_norm
+        self.ffn_norm, self.ffn, self.post_ffn_norm = ffn_norm, ffn, post_ffn_norm
+        self.mixer_conv, self.ffn_conv = mixer_conv, ffn_conv
+
+    def mixers(self) -> List[Mixer]:
+        return [self.mixer]
+
+    def feed_forwards(self) -> List[FeedForward]:
+        return [self.ffn] if self.ffn is not None else []
+
+    def cache_parts(self) -> List[Part]:
+        return [p for p in (self.mixer_conv, self.mixer, self.ffn_conv) if p is not None]
+
+    def parts(self) -> List[Part]:
+        return [p for p in (self.mixer_norm, self.mixer_conv, self.mixer, self.post_mixer_norm, self.ffn_norm, self.ffn_conv,
+                            self.ffn, self.post_ffn_norm) if p is not None]
+
+    def entry_norm(self) -> Optional[Norm]:
+        return self.mixer_norm
+
+    def _read(self, ctx, norm: Norm, conv, x, delta, cache, want_f32: bool):
+        """What a sublayer reads: norm(x + delta), through the convolution when there is one."""
+        dtype = torch.float32 if want_f32 else self.rt.dtype
+        if conv is None:
+            return norm.forward(x, delta, out_dtype=dtype)
+        h = norm.forward(x, delta, out_dtype=torch.float32)
+        mark(ctx, "norm")
+        return conv.forward(ctx, h, cache, out_dtype=dtype)
+
+    @staticmethod
+    def _float_rows(out: torch.Tensor) -> torch.Tensor:
+        """A part's output as one float32 [T, H] tensor (a norm's input)."""
+        if out.dim() == 2 and out.dtype == torch.float32:
+            return out
+        from ..ops import kernels as K
+        return K.sum_parts(out, None, torch.float32)
+
+    def forward(self, ctx: StepContext, x: torch.Tensor, pending, caches):
+        caches = list(caches)
+        conv1_cache = caches.pop(0) if self.mixer_conv is not None else None
+        mixer_cache = caches.pop(0)
+        conv2_cache = caches.pop(0) if self.ffn_conv is not None else None
+        h = self._read(ctx, self.mixer_norm, self.mixer_conv, x, pending, conv1_cache, self.mixer.takes_float32_rows)
+        mark(ctx, "conv" if self.mixer_conv is not None else "norm")
+        a = self._float_rows(self.mixer.forward(ctx, h, mixer_cache))
+        mark(ctx, "mixer")
+        delta = self.post_mixer_norm.forward(a, out_dtype=torch.float32)
+        mark(ctx, "norm")
+        if self.ffn is None:
+            return x, delta
+        h = self._read(ctx, self.ffn_norm, self.ffn_conv, x, delta, conv2_cache, False)
+        mark(ctx, "conv" if self.ffn_conv is not None else "norm")
+        d = self._float_rows(self.ffn.forward(ctx, h))
+        mark(ctx, "feed_forward")
+        delta = self.post_ffn_norm.forward(d, out_dtype=torch.float32)
+        mark(ctx, "norm")
+        return x, delta

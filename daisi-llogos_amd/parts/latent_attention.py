@@ -1,0 +1,109 @@
+"""Attention through a low-rank latent, with a learned sink in the softmax.
+
+    c_q = norm(W_dq h);  q = W_uq c_q                    per head [dim unrotated | rot rotated]
+    [c_raw | k_rot] = W_dkv h;  c = norm(c_raw)          the latent, and one rotated key part for all heads
+    k_h = W_uk,h c;  v_h = W_uv,h c
+    score_h(i, j) = (q_h,plain(i) . k_h(j) + q_h,rot(i) . k_rot(j)) * scale,   j <= i
+    weights = exp(score) / (sum_j exp(score) + exp(sink_h))
+
+Only c and the rotated key part are cached: one row [c | k_rot] a token, for all heads, and no
+values.  The scores are taken in the latent's space, q_h,plain . W_uk,h c = (W_uk,h^T q_h,plain) . c,
+so a head's query becomes [W_uk,h^T q_h,plain | q_h,rot] against the cached row, the weighted sum runs
+over latents, and W_uv,h is applied to that sum."""
+from __future__ import annotations
+
+from typing import Callable, List, Optional
+
+import torch
+
+from ..ops import kernels as K
+from .base import KVSpec, LayerCache, Mixer, Runtime, StepContext, TensorSpec, mark, register_mixer
+from .linear import Linear
+from .rope import Rotary
+
+
+@register_mixer("latent_attention")
+class LatentAttention(Mixer):
+    graph_safe = True
+
+    def __init__(self, prefix: str, hidden: int, n_heads: int, dim: int, rot_dim: int, v_dim: int, q_rank: int,
+                 kv_rank: int, scale: float, eps: float, position: Optional[Rotary] = None, sink: bool = True,
+                 suffix: str = ""):
+        self.prefix, self.hidden = prefix, int(hidden)
+        self.n_heads, self.dim, self.rot_dim, self.v_dim = int(n_heads), int(dim), int(rot_dim), int(v_dim)
+        self.q_rank, self.kv_rank = int(q_rank), int(kv_rank)
+        self.scale, self.eps = float(scale), float(eps)
+        self.position = position
+        self.has_sink = bool(sink)
+        if position is not None and (position.pairing != 1 or position.rot > self.rot_dim):
+            raise ValueError("the rotated key part takes neighbouring pairs, at most rot_dim dimensions")
+        # the cached row [latent | rotated part], widened to the pages' step of 16 dimensions
+        self.row = -(-(self.kv_rank + self.rot_dim) // K.HEAD_DIM_STEP) * K.HEAD_DIM_STEP
+        if self.row > 1024:
+            raise ValueError(f"a cached row of {self.row} values is more than the attention kernel takes (1024)")
+        H = self.n_heads
+        self.dq = Linear([prefix + "dq"], hidden, [self.q_rank], suffix=suffix)
+        self.uq = Linear([prefix + "uq"], self.q_rank, [H * (self.dim + self.rot_dim)], suffix=suffix)
+        self.dkv = Linear([prefix + "dkv"], hidden, [self.kv_rank + self.rot_dim], suffix=suffix)
+        self.o = Linear([prefix + "o"], H * self.v_dim, [hidden], suffix=suffix)
+        self.uk_t = self.uv = self.q_norm_w = self.c_norm_w = self.sink = None
+
+    def _linears(self) -> List[Linear]:
+        return [self.dq, self.uq, self.dkv, self.o]
+
+    @property
+    def head_dim(self) -> int:         # (what Model.step_flops takes as the width of a head's dot products)
+        return self.row
+
+    def kv_spec(self) -> KVSpec:
+        return KVSpec(1, self.row, values=False)
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        p, H = self.prefix, self.n_heads
+        specs = [s for lin in self._linears() for s in lin.tensor_specs()]
+        specs += [TensorSpec(p + "dq.norm", (self.q_rank,), "norm"), TensorSpec(p + "dkv.norm", (self.kv_rank,), "norm"),
+                  TensorSpec(p + "uk", (H * self.dim, self.kv_rank), "matrix"),
+                  TensorSpec(p + "uv", (H * self.v_dim, self.kv_rank), "matrix")]
+        if self.has_sink:
+            specs.append(TensorSpec(p + "sink", (H,), "sink"))
+        return specs
+
+    def bind(self, get: Callable[[str], Optional[torch.Tensor]], rt: Runtime) -> None:
+        super().bind(get, rt)
+        for lin in self._linears():
+            lin.bind(get, rt)
+        H = self.n_heads
+        f32 = lambda name: get(self.prefix + name).to(device=rt.device, dtype=torch.float32).contiguous()
+        self.q_norm_w, self.c_norm_w = f32("dq.norm"), f32("dkv.norm")
+        self.sink = f32("sink") if self.has_sink else None
+        uk = get(self.prefix + "uk").to(device=rt.device, dtype=rt.dtype)
+        # per head the transposed key matrix [rank, dim]: a query's unrotated part times it is the query in the latent's space
+        self.uk_t = uk.view(H, self.dim, self.kv_rank).transpose(1, 2).contiguous()
+        self.uv = get(self.prefix + "uv").to(device=rt.device, dtype=rt.dtype).view(H, self.v_dim, self.kv_rank).contiguous()
+        if self.position is not None and getattr(self.position, "inv_freq", None) is None:
+            self.position.bind(get, rt)
+
+    def matrix_elements(self) -> int:
+        return super().matrix_elements() + self.n_heads * self.kv_rank * (self.dim + self.v_dim)
+
+    def forward(self, ctx: StepContext, h: torch.Tensor, cache: LayerCache) -> torch.Tensor:
+        f32, H, T = torch.float32, self.n_heads, ctx.n_tokens
+        cq = self.dq.forward(h, out_dtype=f32)
+        cq = K.rmsnorm(cq, self.q_norm_w, self.eps, self.rt.dtype)
+        q = self.uq.forward(cq, out_dtype=f32)                                   # [T, H * (dim + rot)]
+        kv = self.dkv.forward(h, out_dtype=f32)                                  # [T, rank + rot]
+        mark(ctx, "projections")
+        cs = self.position.prepare(ctx) if self.position is not None else None
+        qa = torch.empty((T, H, self.row), dtype=self.rt.dtype, device=h.device)
+        K.latent_prepare(ctx, kv, q, qa, self.c_norm_w, self.eps, cs, cache.k_pool, cache.table, H, self.dim, self.rot_dim,
+                         self.position.rot if self.position is not None else 0, self.kv_rank)
+        K.head_products(q.view(T, H, self.dim + self.rot_dim)[:, :, :self.dim], self.uk_t, qa[:, :, :self.kv_rank])
+        mark(ctx, "rotation")
+        lat = K.attention_generic(qa, H * self.row, cache.k_pool, None, cache.table, ctx.tok_seq, ctx.tok_pos, H, 1, self.row,
+                                  self.scale, v_dim=self.kv_rank, head_sink=self.sink)
+        mark(ctx, "attention")
+        a = torch.empty((T, H, self.v_dim), dtype=self.rt.dtype, device=h.device)
+        K.head_products(lat.view(T, H, self.kv_rank), self.uv, a)
+        out = self.o.forward(a.view(T, H * self.v_dim), out_dtype=f32)
+        mark(ctx, "o")
+        return out

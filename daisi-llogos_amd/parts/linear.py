@@ -23,6 +23,7 @@ class Linear(Part):
         self.gated = bool(gated) and len(out_features) == 2 and out_features[0] == out_features[1] \
             and out_features[0] % 16 == 0 and not bias
         self.names = list(names)
+        self.suffix = suffix                             # what a matrix's tensor name has behind its name in `names`
         self.in_features = in_features
         self.out_features = list(out_features)
         self.has_bias = bias
@@ -37,14 +38,14 @@ class Linear(Part):
     def tensor_specs(self) -> List[TensorSpec]:
         specs = []
         for n, o in zip(self.names, self.out_features):
-            specs.append(TensorSpec(n + ".weight", (o, self.in_features), "matrix"))
+            specs.append(TensorSpec(n + self.suffix, (o, self.in_features), "matrix"))
             if self.has_bias:
                 specs.append(TensorSpec(n + ".bias", (o,), "bias"))
         return specs
 
     def bind(self, get: Callable[[str], Optional[torch.Tensor]], rt: Runtime) -> None:
         super().bind(get, rt)
-        mats = [get(n + ".weight") for n in self.names]
+        mats = [get(n + self.suffix) for n in self.names]
         self.weight = _to_device(mats, rt.dtype, rt.device)
         self._pack(rt)
         if self.has_bias:

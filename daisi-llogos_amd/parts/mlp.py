@@ -7,6 +7,9 @@ from typing import Callable, List, Optional
 
 import torch
 
+import math
+
+from ..ops import kernels as K
 from .base import FeedForward, Residual, Runtime, StepContext, TensorSpec, mark, register_feed_forward
 from .linear import Linear
 
@@ -47,5 +50,48 @@ class SwiGLU(FeedForward):
         # otherwise silu(gate) * up is made inside the down product where its kernel can (few rows), by a
         # kernel of its own for many; the residual sum that follows adds the product's parts
         out = self.down.product(gu, swiglu_input=True, f32_ok=True)
+        mark(ctx, "down")
+        return out
+
+
+def _softplus(z: float) -> float:
+    return math.log1p(math.exp(-abs(z))) + max(z, 0.0)
+
+
+@register_feed_forward("activated")
+class ActivatedMLP(FeedForward):
+    """d = W_down act(W_up h) with an activation from ops.kernels.ACTIVATIONS.  'xielu' has two learned
+    numbers (p, q) in the tensor `prefix + "act"`: z > 0: softplus(p) z^2 + z / 2; z <= 0:
+    (1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2; the two softplus values are worked out once, when
+    the tensor is bound."""
+    graph_safe = True
+
+    def __init__(self, prefix: str, hidden: int, intermediate: int, activation: str = "xielu", suffix: str = ""):
+        if activation not in K.ACTIVATIONS:
+            raise ValueError(f"unknown activation '{activation}'; known: {sorted(K.ACTIVATIONS)}")
+        self.prefix, self.hidden, self.intermediate, self.activation = prefix, int(hidden), int(intermediate), activation
+        self.up = Linear([prefix + "up"], hidden, [intermediate], suffix=suffix)
+        self.down = Linear([prefix + "down"], intermediate, [hidden], suffix=suffix)
+        self.a = self.b = 0.0
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        specs = self.up.tensor_specs() + self.down.tensor_specs()
+        if self.activation == "xielu":
+            specs.append(TensorSpec(self.prefix + "act", (2,), "shape"))
+        return specs
+
+    def bind(self, get: Callable[[str], Optional[torch.Tensor]], rt: Runtime) -> None:
+        super().bind(get, rt)
+        self.up.bind(get, rt)
+        self.down.bind(get, rt)
+        if self.activation == "xielu":
+            p, q = (float(v) for v in get(self.prefix + "act").to(torch.float32).reshape(-1).tolist())
+            self.a, self.b = _softplus(p), 0.5 + _softplus(q)
+
+    def forward(self, ctx: StepContext, h):
+        z = self.up.product(h, f32_ok=True)
+        mark(ctx, "up")
+        act = K.activation(z, self.activation, self.rt.dtype, self.a, self.b)
+        out = self.down.forward(act, out_dtype=torch.float32)
         mark(ctx, "down")
         return out

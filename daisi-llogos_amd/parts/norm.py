@@ -16,28 +16,35 @@ from .base import Norm, NormedRows, Runtime, TensorSpec, register_norm
 class RMSNorm(Norm):
     takes_row_squares = True
 
-    def __init__(self, name: str, width: int, eps: float):
+    def __init__(self, name: str, width: int, eps: float, offset: float = 0.0, suffix: str = ".weight"):
+        """offset: the stored tensor is the weight less this number (1 for checkpoints that keep
+        their norm weights around zero); the sum is made once, in float32, when the tensor is bound.
+        suffix: what the tensor's name has behind `name`."""
         self.name = name
         self.width = width
         self.eps = float(eps)
+        self.offset = float(offset)
+        self.suffix = suffix
         self.weight: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> List[TensorSpec]:
-        return [TensorSpec(self.name + ".weight", (self.width,), "norm")]
+        return [TensorSpec(self.name + self.suffix, (self.width,), "offset" if self.offset else "norm")]
 
     def bind(self, get: Callable[[str], Optional[torch.Tensor]], rt: Runtime) -> None:
         super().bind(get, rt)
-        self.weight = get(self.name + ".weight").to(device=rt.device, dtype=torch.float32).contiguous()
+        self.weight = get(self.name + self.suffix).to(device=rt.device, dtype=torch.float32).contiguous()
+        if self.offset:
+            self.weight += self.offset
 
     def forward(self, x: torch.Tensor, delta=None, rows: Optional[torch.Tensor] = None,
-                write_back: bool = True, lazy: bool = False):
+                write_back: bool = True, lazy: bool = False, out_dtype: Optional[torch.dtype] = None):
         if isinstance(delta, K.RowSquares):
             # the product before has added itself to x; if it also left this norm's rows without their
             # scale, a consumer that takes them needs no kernel here
             if lazy and rows is None and delta.unscaled is not None and delta.norm_w is self.weight:
                 return NormedRows(delta, self.eps, self, x)
             delta = None
-        return K.rmsnorm(x, self.weight, self.eps, self.rt.dtype, delta=delta, rows=rows, write_back=write_back)
+        return K.rmsnorm(x, self.weight, self.eps, out_dtype or self.rt.dtype, delta=delta, rows=rows, write_back=write_back)
 
     def row_weight(self) -> Optional[torch.Tensor]:
         return self.weight

@@ -38,6 +38,29 @@ def llama3_factors(freqs: List[float], factor: float, low_freq_factor: float, hi
     return out
 
 
+def yarn_frequencies(freqs: List[float], rot: int, theta: float, factor: float, original: float,
+                     fast: float, slow: float) -> List[float]:
+    """YaRN: pairs that turn more than `fast` times over the original context keep their
+    frequency, pairs that turn fewer than `slow` times are slowed by `factor`, and the pairs
+    between are mixed along a ramp over the pair index.  A pair index as a function of turns t is
+    rot * ln(original / (2 pi t)) / (2 ln theta); the ramp runs from the floor of that at `fast`
+    to its ceiling at `slow`, both kept within 0 .. rot - 1."""
+    def pair_at(turns: float) -> float:
+        return rot * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(theta))
+    lo = max(math.floor(pair_at(fast)), 0)
+    hi = min(math.ceil(pair_at(slow)), rot - 1)
+    out = []
+    for i, f in enumerate(freqs):
+        ramp = min(1.0, max(0.0, (i - lo) / max(hi - lo, 0.001)))
+        out.append(f / factor * ramp + f * (1.0 - ramp))
+    return out
+
+
+def yarn_amplitude(factor: float) -> float:
+    """What YaRN multiplies cos and sin with."""
+    return 0.1 * math.log(factor) + 1.0
+
+
 @register_position("rotary")
 class Rotary(PositionEncoding):
     def __init__(self, head_dim: int, rot: int, theta: float, pairing: str = "split_half",
@@ -50,6 +73,7 @@ class Rotary(PositionEncoding):
         self.rot = rot
         self.theta = float(theta)
         self.pairing = SPLIT_HALF if pairing == "split_half" else INTERLEAVED
+        self.amplitude = 1.0                 # cos and sin are multiplied by this
         freqs = inverse_frequencies(rot, theta)
         if scaling:
             kind = scaling.get("rope_type", scaling.get("type"))
@@ -59,6 +83,10 @@ class Rotary(PositionEncoding):
                 freqs = [f / c for f, c in zip(freqs, fac)]
             elif kind == "linear":
                 freqs = [f / float(scaling["factor"]) for f in freqs]
+            elif kind == "yarn":
+                freqs = yarn_frequencies(freqs, rot, self.theta, float(scaling["factor"]), float(scaling["original"]),
+                                         float(scaling["fast"]), float(scaling["slow"]))
+                self.amplitude = yarn_amplitude(float(scaling["factor"]))
             elif kind not in (None, "default"):
                 raise ValueError(f"unknown rotary scaling '{kind}'")
         self.freqs = freqs
@@ -73,6 +101,6 @@ class Rotary(PositionEncoding):
         key = ("rotary", id(self))
         table = ctx.shared.get(key)
         if table is None:
-            table = K.rope_table(ctx.tok_pos, self.inv_freq)
+            table = K.rope_table(ctx.tok_pos, self.inv_freq, self.amplitude)
             ctx.shared[key] = table
         return table

@@ -20,6 +20,11 @@ from .safetensors_io import write_safetensors
 _STORE = {"bfloat16": torch.bfloat16, "float32": torch.float32, "float16": torch.float16}
 
 
+# kinds of tensors that are drawn uniformly from a range instead of N(0, std): norm weights around
+# one, norm weights stored as offsets from one, mixing weights between 0 and 1, decay biases (the
+# decay is exp(-exp(bias + ...))), learned scores of a softmax sink, an activation's shape numbers
+_UNIFORM = {"norm": (0.9, 1.1), "offset": (-0.1, 0.1), "unit": (0.0, 0.8), "decay": (-6.0, -0.5), "sink": (0.0, 4.0),
+            "shape": (-1.5, 0.5), "taps": (-0.5, 0.5), "bonus": (-0.5, 1.5)}
 _MASK32 = 0xFFFFFFFF
 _CHUNK = {"cpu": 1 << 20, "cuda": 1 << 26}     # elements made at a time (on the CPU what stays in the caches)
 
@@ -41,13 +46,14 @@ def _mix32(x: torch.Tensor) -> torch.Tensor:
 
 def _random_chunk(first: int, count: int, keys: Tuple[int, int], kind: str, std: float, device) -> torch.Tensor:
     """Values of elements first .. first + count - 1 of a tensor, float64: a counter-based
-    stream, element i's value depends on (keys, i) alone.  'norm': 1 + U(-0.1, 0.1); anything
+    stream, element i's value depends on (keys, i) alone.  'norm': 1 + U(-0.1, 0.1), and the other uniform kinds of _UNIFORM; anything
     else N(0, std) by Box-Muller from two 24-bit uniforms."""
     idx = torch.arange(first, first + count, dtype=torch.int64, device=device)
     a = _mix32(_mix32((idx + keys[0]) & _MASK32) ^ keys[1])
     u1 = (a >> 8).to(torch.float64)
-    if kind == "norm":
-        return 1.0 + (u1 * (0.2 / (1 << 24)) - 0.1)
+    if kind in _UNIFORM:
+        lo, hi = _UNIFORM[kind]
+        return lo + u1 * ((hi - lo) / (1 << 24))
     b = _mix32(a ^ 0x9E3779B9)
     u2 = (b >> 8).to(torch.float64) * (1.0 / (1 << 24))
     radius = torch.sqrt(-2.0 * torch.log((u1 + 1.0) * (1.0 / (1 << 24))))          # u in (0, 1]
