@@ -37,14 +37,14 @@ def nipulorn_spec(cfg: NipulornConfig) -> ModelSpec:
                                               v_dim=m.vdim, q_rank=m.q_rank, kv_rank=m.kv_rank, scale=m.scale, eps=eps,
                                               position=position))
         more = {"post_mixer_norm": ("norm",) + norm(p + "norm1b")}
-        if cfg.canon_taps > 1:
+        if cfg.canon_taps >= 1:
             more["mixer_conv"] = ("part", "causal_conv", dict(name=p + "canon1", width=W, taps=cfg.canon_taps))
         spec = LayerSpec(mixer=mixer, mixer_norm=norm(p + "norm1"), block="sandwich", more=more)
         if L.mlp is not None:
             spec.ffn = ("activated", dict(prefix=p + "mlp.", hidden=W, intermediate=L.mlp.ff, activation="xielu"))
             spec.ffn_norm = norm(p + "norm2")
             more["post_ffn_norm"] = ("norm",) + norm(p + "norm2b")
-            if cfg.canon_taps > 1:
+            if cfg.canon_taps >= 1:
                 more["ffn_conv"] = ("part", "causal_conv", dict(name=p + "canon2", width=W, taps=cfg.canon_taps))
         layers.append(spec)
     return ModelSpec(vocab_size=cfg.vocab, hidden_size=W, embed_name="embed", layers=layers,

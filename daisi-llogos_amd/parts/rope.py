@@ -84,6 +84,9 @@ class Rotary(PositionEncoding):
             elif kind == "linear":
                 freqs = [f / float(scaling["factor"]) for f in freqs]
             elif kind == "yarn":
+                lacking = [k for k in ("factor", "original", "fast", "slow") if k not in scaling]
+                if lacking:
+                    raise ValueError(f"rotary scaling 'yarn' needs {', '.join(lacking)}")
                 freqs = yarn_frequencies(freqs, rot, self.theta, float(scaling["factor"]), float(scaling["original"]),
                                          float(scaling["fast"]), float(scaling["slow"]))
                 self.amplitude = yarn_amplitude(float(scaling["factor"]))

@@ -1,0 +1,170 @@
+"""The Nipulorn design without a GPU: its configuration reader, the model description built from
+it, the cache units it asks for, the rotary scaling rule against numbers worked by hand, and the
+plain implementation's own consistency (a recurrence or a convolution continued from a carried
+state equals the whole sequence)."""
+import copy
+import importlib
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import nipulorn_configs as nc
+import plain_nipulorn as pn
+
+L = importlib.import_module("daisi-llogos_amd")
+reg = importlib.import_module("daisi-llogos_amd.config.registry")
+ncfg = importlib.import_module("daisi-llogos_amd.config.nipulorn_config")
+rope = importlib.import_module("daisi-llogos_amd.parts.rope")
+P = importlib.import_module("daisi-llogos_amd.parts")
+
+
+def _model(cfg):
+    arch = reg.architecture_of(cfg)
+    assert arch.name == "Nipulorn" and arch.reads_shapes
+    return L.Model(arch.model_spec(arch.read_config(cfg)))
+
+
+def test_the_registry_finds_the_design_by_a_string_or_a_list():
+    assert reg.architecture_of({"architecture": "Nipulorn"}).name == "Nipulorn"
+    assert reg.architecture_of({"architectures": ["Nipulorn"]}).name == "Nipulorn"
+    with pytest.raises(L.ConfigError, match="unknown architecture"):
+        reg.architecture_of({"architecture": "Nipulorn2"})
+
+
+def test_every_size_and_constant_comes_from_the_file():
+    c = ncfg.NipulornConfig.from_dict(nc.NIP_A)
+    assert (c.vocab, c.width, c.embedding_scale, c.logit_scale, c.norm_eps, c.canon_taps) == (211, 96, 4.0, 0.25, 1e-6, 3)
+    a, w, b, w2 = c.layers
+    assert (a.type, a.mixer.heads, a.mixer.dim, a.mixer.rot_dim, a.mixer.vdim, a.mixer.q_rank, a.mixer.kv_rank) == \
+        ("latent_attention", 3, 32, 8, 24, 40, 48)
+    assert a.mixer.rot_scaling == ncfg.YarnScaling(4.0, 48.0, 8.0, 1.5) and a.mlp.ff == 160 and a.mixer.scale == 0.35
+    assert (w.type, w.mixer.heads, w.mixer.dim, w.mixer.decay_rank, w.mlp.ff) == ("wkv", 2, 40, 12, 128)
+    assert b.mixer.rot_dims == 8 and b.mixer.rot_dim == 16 and b.mixer.rot_scaling is None and b.mlp is None
+    assert w2.mlp is None
+
+
+def test_the_decay_rank_is_a_tensors_first_dimension_when_the_file_does_not_give_it():
+    cfg = copy.deepcopy(nc.NIP_A)
+    del cfg["layers"][1]["mixer"]["decay_rank"]
+    assert ncfg.NipulornConfig.from_dict(cfg, shapes={"l1.mix.w1": (7, 96)}).layers[1].mixer.decay_rank == 7
+    assert ncfg.NipulornConfig.from_dict(cfg).layers[1].mixer.decay_rank == 16          # nothing to go by: a default
+
+
+@pytest.mark.parametrize("change,match", [
+    (lambda c: c.pop("width"), "width"), (lambda c: c["norm"].pop("eps"), "eps"),
+    (lambda c: c["layers"][0].update(type="conv"), "unknown layer type"),
+    (lambda c: c["layers"][0]["mixer"].pop("kv_rank"), "kv_rank"),
+    (lambda c: c["layers"][0]["mlp"].update(kind="routed"), "feed-forward kind"),
+    (lambda c: c["layers"][0]["mixer"]["rot"].update(dims=7), "rot.dims"),
+    (lambda c: c.update(layers=[]), "layers"),
+])
+def test_a_file_that_cannot_describe_a_model_names_the_key(change, match):
+    cfg = copy.deepcopy(nc.NIP_A)
+    change(cfg)
+    with pytest.raises(L.ConfigError, match=match):
+        ncfg.NipulornConfig.from_dict(cfg)
+
+
+def test_the_model_asks_for_the_designs_tensors_and_cache_units():
+    m = _model(nc.NIP_A)
+    names = {s.name: tuple(s.shape) for s in m.tensor_specs()}
+    assert names["embed"] == (211, 96) and names["final.norm"] == (96,) and "lm_head.weight" not in names
+    assert names["l0.mix.dkv"] == (48 + 8, 96) and names["l0.mix.uq"] == (3 * 40, 40) and names["l0.mix.uk"] == (96, 48)
+    assert names["l0.mix.uv"] == (72, 48) and names["l0.mix.sink"] == (3,) and names["l0.mix.dq.norm"] == (40,)
+    assert names["l0.mlp.act"] == (2,) and names["l0.canon2"] == (96, 3) and names["l0.norm2b"] == (96,)
+    assert names["l1.mix.w1"] == (12, 96) and names["l1.mix.w2"] == (80, 12) and names["l1.mix.u"] == (2, 40)
+    assert names["l1.mix.mu.w"] == (96,) and names["l1.mix.o"] == (96, 80)
+    assert "l2.norm2" not in names and "l2.canon2" not in names and "l3.mlp.up" not in names
+    # per layer: the mixer's convolution, the mixer, and the feed-forward's convolution where there is one
+    needs = m.cache_needs()
+    assert len(needs) == 3 + 3 + 2 + 2
+    conv = P.StateSpec((2, 96), torch.float32)
+    assert needs[0] == (None, conv) and needs[2] == (None, conv)
+    assert needs[1] == (P.KVSpec(1, 64, values=False), None)                      # 48 + 8 widened to a multiple of 16
+    assert needs[4] == (None, P.StateSpec((2 * 40 * 40 + 96,), torch.float32))
+    assert needs[7] == (P.KVSpec(1, 48, values=False), None)                      # 20 + 16
+    assert m.graph_safe and m.spec.tie_head and m.spec.embed_scale == 4.0 and m.spec.logit_scale == 0.25
+
+
+def test_a_cache_without_a_device_counts_the_units(tmp_path):
+    m = _model(nc.NIP_B)
+    cache = L.Cache(m.cache_needs(), m.cache_reads(), 256, None, n_slots=2)
+    assert len(cache.groups) == 1 and len(cache.groups[0].entries) == 2           # two latent layers with equal rows share pages
+    s = cache.alloc_slot()
+    cache.reserve([s], [70])
+    cache.commit([s], [70])
+    assert cache.free_pages() == [2]
+    cache.free_slot(s)
+    assert cache.free_pages() == [4]
+
+
+def test_yarn_frequencies_by_hand():
+    # 8 rotated dimensions, base 100: f = 1, 100^-0.25, 100^-0.5, 100^-0.75
+    f = rope.inverse_frequencies(8, 100.0)
+    assert np.allclose(f, [1.0, 10 ** -0.5, 0.1, 10 ** -1.5])
+    # pair index at t turns over the original 64 positions: 8 ln(64 / (2 pi t)) / (2 ln 100)
+    at = lambda t: 8 * math.log(64 / (2 * math.pi * t)) / (2 * math.log(100.0))
+    lo, hi = max(math.floor(at(4.0)), 0), min(math.ceil(at(1.0)), 7)
+    assert (lo, hi) == (0, 3) and abs(at(1.0) - 2.0160) < 1e-3
+    got = rope.yarn_frequencies(f, 8, 100.0, factor=2.0, original=64.0, fast=4.0, slow=1.0)
+    ramp = [0.0, 1 / 3, 2 / 3, 1.0]
+    assert np.allclose(got, [x / 2.0 * r + x * (1 - r) for x, r in zip(f, ramp)])
+    assert abs(rope.yarn_amplitude(2.0) - (0.1 * math.log(2.0) + 1.0)) < 1e-15
+    r = P.Rotary(16, 8, 100.0, pairing="interleaved", scaling=dict(type="yarn", factor=2.0, original=64, fast=4.0, slow=1.0))
+    assert np.allclose(r.freqs, got) and r.amplitude == rope.yarn_amplitude(2.0)
+    fp, amp = pn.yarn_frequencies(8, 100.0, {"factor": 2.0, "original": 64, "fast": 4.0, "slow": 1.0})
+    assert np.allclose(fp, got) and amp == r.amplitude
+    # a ramp of no width: lo == hi, the divisor's floor keeps the step at that pair
+    got = rope.yarn_frequencies(f, 8, 100.0, factor=3.0, original=64.0, fast=1.0, slow=1.0)
+    assert np.allclose(got, [f[0], f[1], f[2], f[3] / 3.0]) or np.allclose(got[:2], f[:2])
+
+
+def test_plain_recurrence_and_convolution_continue_from_a_carried_state():
+    rng = np.random.default_rng(0)
+    T, H, D = 23, 2, 5
+    r, k, v = (rng.standard_normal((T, H, D)) for _ in range(3))
+    w = rng.uniform(0.3, 0.99, (T, H, D))
+    u = rng.standard_normal((H, D))
+    whole, S = pn.wkv_recurrence(r, k, v, w, u)
+    a, Sa = pn.wkv_recurrence(r[:9], k[:9], v[:9], w[:9], u)
+    b, Sb = pn.wkv_recurrence(r[9:], k[9:], v[9:], w[9:], u, Sa)
+    assert np.allclose(np.concatenate([a, b]), whole) and np.allclose(Sb, S)
+    # the first token sees the bonus alone: o_0 = (sum_i r_i u_i k_i) v
+    assert np.allclose(whole[0, 0], (r[0, 0] * u[0] * k[0, 0]).sum() * v[0, 0])
+    h, cw = rng.standard_normal((T, 4)), rng.standard_normal((4, 3))
+    out = pn.input_convolution(h, cw)
+    assert np.allclose(out[0], h[0] + cw[:, 2] * h[0]) and np.allclose(out[2], h[2] + cw[:, 0] * h[0] + cw[:, 1] * h[1] + cw[:, 2] * h[2])
+    assert np.allclose(pn.token_shift(h, np.full(4, 0.25))[0], 0.75 * h[0])
+    assert np.allclose(pn.token_shift(h[5:], np.full(4, 0.25), before=h[4]), pn.token_shift(h, np.full(4, 0.25))[5:])
+
+
+def test_plain_activation_and_sink_by_hand():
+    sp = lambda z: math.log(1 + math.exp(z))
+    assert np.allclose(pn.xielu(np.array([2.0, -1.0, 0.0]), 0.3, -0.7),
+                       [sp(0.3) * 4 + 1.0, (0.5 + sp(-0.7)) * (math.exp(-1) - 1 + 1) - 0.5, 0.0])
+    assert abs(pn.gelu_tanh(np.float64(1.0)) - 0.8411919906) < 1e-9
+    # one key with score 0 and a sink of 0: the value gets half the weight
+    assert np.allclose(pn.sink_softmax_attention(np.zeros((1, 1)), np.array([[2.0, 4.0]]), 0.0), [[1.0, 2.0]])
+    # a sink far below the scores changes nothing
+    s, v = np.array([[0.0, 9.0], [1.0, 2.0]]), np.array([[1.0], [3.0]])
+    e = math.exp(1.0) / (math.exp(1.0) + math.exp(2.0))
+    assert np.allclose(pn.sink_softmax_attention(s, v, -50.0), [[1.0], [e * 1 + (1 - e) * 3]])
+
+
+def test_random_models_of_the_design_are_written_and_fit_their_description(tmp_path):
+    loader = importlib.import_module("daisi-llogos_amd.weights.loader")
+    for name, cfg in nc.ALL.items():
+        path = L.write_random_model(str(tmp_path / name), cfg, seed=3)
+        ck = loader.Checkpoint(path)
+        arch = reg.architecture_of(cfg)
+        m = L.Model(arch.model_spec(arch.read_config(cfg, shapes=ck.shapes())))
+        ck.check(m.tensor_specs(), tied_head="embed.weight")
+        mu = ck.get("l0.mix.mu.r") if cfg["layers"][0]["type"] == "wkv" else None
+        if mu is not None:
+            assert 0.0 <= float(mu.min()) and float(mu.max()) <= 0.8
+        ck.close()
+        c2, w = pn.load_folder(path)
+        assert np.isfinite(pn.forward(c2, w, [1, 2, 3, 4, 5])).all()
