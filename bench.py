@@ -140,8 +140,107 @@ def clocks_under_load(torch, K, seconds=3.0):
     under("the library's gate/up product of 2,048 rows", lambda: torch.matmul(a, w.t()), flops)
 
 
+# ---------------------------------------------------------------------------------------------
+# --design nipulorn: the Nipulorn design beside the dense decoder at equal width, depth and weight
+# ---------------------------------------------------------------------------------------------
+def nipulorn_config(width, layers, vocab, ff):
+    """Layers of real sizes: three recurrent layers to one of latent attention, a feed-forward behind each;
+    heads of 64 channels in the recurrence; attention with 128 + 64 query/key dimensions a head, values of 128,
+    a latent of 512 for keys and values and of 3 * width / 8 for queries."""
+    heads = width // 128
+    wkv = {"type": "wkv", "mixer": {"heads": width // 64, "dim": 64, "decay_rank": 64}, "mlp": {"kind": "dense", "ff": ff}}
+    lat = {"type": "latent_attention",
+           "mixer": {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "q_rank": 3 * width // 8, "kv_rank": 512,
+                     "scale": 192 ** -0.5, "rot": {"base": 10000.0, "dims": 64,
+                                                   "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}},
+           "mlp": {"kind": "dense", "ff": ff}}
+    return {"architecture": "Nipulorn", "vocab": vocab, "width": width, "embedding": {"scale": 1.0}, "logit_scale": 1.0,
+            "norm": {"eps": 1e-5}, "canon": {"taps": 4}, "layers": [lat if i % 4 == 3 else wkv for i in range(layers)],
+            "torch_dtype": "bfloat16"}
+
+
+def compare_designs(args) -> int:
+    """Prefill and decode throughput of Nipulorn models of real layer sizes (random weights) and of the dense
+    decoder with the same width, depth and about the same weight bytes, and where a step's time goes part by
+    part in both.  One JSON line at the end."""
+    import numpy as np
+    import torch
+    llogos = importlib.import_module("daisi-llogos_amd")
+    rng = np.random.default_rng(0)
+    sizes = [("2048 wide", 2048, 8192, 8), ("4096 wide", 4096, 14336, 8)]
+    record = {"metric": "design_comparison", "design": "Nipulorn", "against": "dense decoder (Llama sizes)", "dtype": "bf16",
+              "data": "synthetic", "sizes": []}
+
+    def measure(label, cfg, vocab):
+        eng = llogos.Engine.from_config(cfg, seed=0, dtype="bfloat16", max_tokens=8 * 1024 + args.prefill_tokens + 256, n_slots=8)
+        model = eng.model
+        out = {"weights_GB": round(model.step_weight_bytes() / 1e9, 3)}
+        toks = lambda n: [int(t) for t in rng.integers(0, vocab, size=n)]
+
+        def timed(fn, repeat=3):
+            best = 1e9
+            for _ in range(repeat):
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                fn()
+                torch.cuda.synchronize()
+                best = min(best, time.perf_counter() - t0)
+            return best
+
+        def prompt():
+            s = eng.alloc_slot()
+            eng.step([(s, toks(args.prefill_tokens))], want="last")
+            eng.free_slot(s)
+        prompt()
+        dt = timed(prompt)
+        out["prefill_tok_s"] = round(args.prefill_tokens / dt)
+        out["prefill_ms"] = round(dt * 1e3, 2)
+        probe = llogos.StepProbe()
+        s = eng.alloc_slot()
+        probe.hold()
+        probe.start()
+        eng.step([(s, toks(args.prefill_tokens))], want="last", probe=probe)
+        eng.free_slot(s)
+        out["prefill_parts_us"] = {k: round(v, 1) for k, v in probe.microseconds_per_call().items()}
+        for batch in (1, 8):
+            slots = [eng.alloc_slot() for _ in range(batch)]
+            eng.step([(x, toks(args.prompt_len)) for x in slots], want="last")
+            step = lambda: eng.step([(x, [1]) for x in slots], want="last", borrow=True)
+            for _ in range(args.warmup):
+                step()
+            dt = timed(lambda: [step() for _ in range(args.steps)], repeat=2) / args.steps
+            out[f"decode_b{batch}_tok_s"] = round(batch / dt)
+            out[f"decode_b{batch}_us"] = round(dt * 1e6, 1)
+            out[f"decode_b{batch}_roofline"] = round(model.step_weight_bytes() / HBM_PEAK / dt, 3)
+            if batch == 8:
+                probe = llogos.StepProbe()
+                probe.hold()
+                probe.start()
+                eng.step([(x, [1]) for x in slots], want="last", probe=probe)
+                out["decode_b8_parts_us"] = {k: round(v, 1) for k, v in probe.microseconds_per_call().items()}
+            for x in slots:
+                eng.free_slot(x)
+        print(f"[design] {label}: {json.dumps(out)}", file=sys.stderr, flush=True)
+        del eng
+        torch.cuda.empty_cache()
+        return out
+
+    vocab = 32000
+    for name, width, ff, layers in sizes:
+        dense = dict(LLAMA31_8B, hidden_size=width, intermediate_size=ff, num_hidden_layers=layers, vocab_size=vocab,
+                     num_attention_heads=width // 128, num_key_value_heads=max(1, width // 512), tie_word_embeddings=True)
+        # two matrices a feed-forward instead of three: half as wide again for the same weight
+        nip = nipulorn_config(width, layers, vocab, ff * 3 // 2)
+        record["sizes"].append({"size": name, "layers": layers, "nipulorn": measure(f"nipulorn {name}", nip, vocab),
+                                "dense": measure(f"dense {name}", dense, vocab)})
+    print(json.dumps(record), flush=True)
+    return 0
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser()
+    ap.add_argument("--design", choices=["nipulorn"], default=None,
+                    help="instead of the default run: this design beside the dense decoder at equal sizes (prefill, decode, parts)")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=248)   # + 8 warm-up = 256 new tokens
     ap.add_argument("--warmup", type=int, default=8)
@@ -159,6 +258,10 @@ def main(argv=None) -> int:
     ap.add_argument("--top-p", type=float, default=0.9)
     args = ap.parse_args(argv)
     prefill_tokens = args.prefill_tokens
+    if args.design:
+        if args.steps == 248:
+            args.steps = 64
+        return compare_designs(args)
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU library")
         return 2

@@ -14,10 +14,12 @@
 // (2i, 2i + 1) by the table cs [T, rot_dims / 2] of (cos, sin), the rest pass unchanged.
 // qfull [T, ldq] float holds per head [dim | rot]; the head's rot part is rotated the same way
 // and written to q_out[t, h, rank .. rank + rot), zeros behind it up to hd.
+// With a value pool (the matrix cores' attention reads values in their own operand order) the
+// latent is stored there too, as dimensions 0..rank-1 of the token's value row.
 template <typename T>
 __global__ void latent_prepare_kernel(const float* __restrict__ kv, int ldkv, const float* __restrict__ qfull, int ldq,
                                       T* __restrict__ q_out, const float* __restrict__ norm_w, float eps,
-                                      const float2* __restrict__ cs, T* __restrict__ k_pool, PagedKV cache,
+                                      const float2* __restrict__ cs, T* __restrict__ k_pool, T* __restrict__ v_pool, PagedKV cache,
                                       const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
                                       int n_heads, int dim, int rot, int rot_dims, int rank, int hd) {
     __shared__ float red[16];
@@ -26,14 +28,18 @@ __global__ void latent_prepare_kernel(const float* __restrict__ kv, int ldkv, co
     const float* row = kv + (size_t)t * ldkv;
     const int half = rot_dims / 2;
     const float2* tab = cs + (size_t)t * half;
-    T* page = k_pool + paged_base(cache, seq, 0, pos);
+    const size_t page_at = paged_base(cache, seq, 0, pos);
+    T* page = k_pool + page_at;
     const int in_page = pos % kPageTokens;
 
     float ss = 0.f;
     for (int i = tid; i < rank; i += blockDim.x) ss = fmaf(row[i], row[i], ss);
     const float inv = 1.0f / sqrtf(block_sum(ss, red) / (float)rank + eps);
-    for (int i = tid; i < rank; i += blockDim.x)
-        store_f32(page + page_key_offset(in_page, i, hd), row[i] * inv * norm_w[i]);
+    for (int i = tid; i < rank; i += blockDim.x) {
+        const float v = row[i] * inv * norm_w[i];
+        store_f32(page + page_key_offset(in_page, i, hd), v);
+        if (v_pool) store_f32(v_pool + page_at + page_value_offset(in_page, i), v);     // the latent again, as a value
+    }
     for (int i = tid; i < hd - rank; i += blockDim.x) {
         float v = 0.f;
         if (i < rot) {
@@ -64,7 +70,7 @@ __global__ void latent_prepare_kernel(const float* __restrict__ kv, int ldkv, co
 }
 
 LLOGOS_EXPORT int llogos_latent_prepare(const float* kv, int ldkv, const float* qfull, int ldq, void* q_out, int dtype,
-                                        const float* norm_w, float eps, const void* cs, void* k_pool,
+                                        const float* norm_w, float eps, const void* cs, void* k_pool, void* v_pool,
                                         const int* table, int table_stride, const int* tok_seq, const int* tok_pos,
                                         int T, int n_heads, int dim, int rot, int rot_dims, int rank, int hd,
                                         hipStream_t stream) {
@@ -73,10 +79,10 @@ LLOGOS_EXPORT int llogos_latent_prepare(const float* kv, int ldkv, const float* 
     PagedKV cache{table, table_stride, 1, hd};
     if (dtype == DT_F32)
         latent_prepare_kernel<float><<<T, 256, 0, stream>>>(kv, ldkv, qfull, ldq, (float*)q_out, norm_w, eps, (const float2*)cs,
-                                                            (float*)k_pool, cache, tok_seq, tok_pos, n_heads, dim, rot, rot_dims, rank, hd);
+                                                            (float*)k_pool, (float*)v_pool, cache, tok_seq, tok_pos, n_heads, dim, rot, rot_dims, rank, hd);
     else if (dtype == DT_BF16)
         latent_prepare_kernel<bf16_t><<<T, 256, 0, stream>>>(kv, ldkv, qfull, ldq, (bf16_t*)q_out, norm_w, eps, (const float2*)cs,
-                                                             (bf16_t*)k_pool, cache, tok_seq, tok_pos, n_heads, dim, rot, rot_dims, rank, hd);
+                                                             (bf16_t*)k_pool, (bf16_t*)v_pool, cache, tok_seq, tok_pos, n_heads, dim, rot, rot_dims, rank, hd);
     else
         return LLOGOS_BAD_ARGUMENT;
     return LLOGOS_LAUNCH_CHECK();

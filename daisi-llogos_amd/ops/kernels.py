@@ -395,12 +395,13 @@ def activation(x: torch.Tensor, kind: str, out_dtype: torch.dtype, a: float = 0.
 # attention through a latent
 # ----------------------------------------------------------------------------
 def latent_prepare(ctx, kv: torch.Tensor, qfull: torch.Tensor, q_out: torch.Tensor, norm_w: torch.Tensor, eps: float,
-                   cs: Optional[torch.Tensor], k_pool: torch.Tensor, table: torch.Tensor, n_heads: int, dim: int, rot: int,
-                   rot_dims: int, rank: int) -> None:
+                   cs: Optional[torch.Tensor], k_pool: torch.Tensor, v_pool: Optional[torch.Tensor], table: torch.Tensor,
+                   n_heads: int, dim: int, rot: int, rot_dims: int, rank: int) -> None:
     """From kv float32 [T, rank + rot] and qfull float32 [T, heads * (dim + rot)]: the normed latent and
     the rotated shared key part go to the token's key row in the cache ([rank | rot | zeros]); each
-    head's rotated query part goes to q_out[t, h, rank:] ([T, heads, hd], hd the cache's row width)."""
-    _dev(kv, qfull, q_out, norm_w, cs, k_pool, table, ctx.tok_seq, ctx.tok_pos)
+    head's rotated query part goes to q_out[t, h, rank:] ([T, heads, hd], hd the cache's row width).  With a
+    value pool the latent is also stored as the token's value row."""
+    _dev(kv, qfull, q_out, norm_w, cs, k_pool, v_pool, table, ctx.tok_seq, ctx.tok_pos)
     _i32(table, "table")
     T = ctx.n_tokens
     hd = q_out.shape[-1]
@@ -408,15 +409,63 @@ def latent_prepare(ctx, kv: torch.Tensor, qfull: torch.Tensor, q_out: torch.Tens
     _need(qfull.dtype == torch.float32 and qfull.shape == (T, n_heads * (dim + rot)), "latent_prepare: q must be float32 [T, heads * (dim + rot)]")
     _need(q_out.shape == (T, n_heads, hd) and q_out.dtype == k_pool.dtype, "latent_prepare: q_out must be [T, heads, hd] of the cache's type")
     _need(hd % 16 == 0 and hd >= rank + rot, "latent_prepare: the cache's row is too narrow")
-    _check_pools(k_pool, None, 1, hd, "latent_prepare")
+    _check_pools(k_pool, v_pool, 1, hd, "latent_prepare")
+    _need(v_pool is None or v_pool.dtype == k_pool.dtype, "latent_prepare: the pools' types differ")
     _need(norm_w.dtype == torch.float32 and norm_w.shape == (rank,), "latent_prepare: norm weight must be float32 [rank]")
     _need(rot_dims % 2 == 0 and 0 <= rot_dims <= rot, "latent_prepare: rotated dimensions must be even and within rot")
     if rot_dims:
         _need(cs is not None and cs.dtype == torch.float32 and cs.shape == (T, rot_dims // 2, 2), "latent_prepare: rotary table shape")
     _need(table.dim() == 2, "latent_prepare: page table must be [batch, pages]")
     _check(_lib().llogos_latent_prepare(_p(kv), kv.stride(0), _p(qfull), qfull.stride(0), _p(q_out), _dt(q_out), _p(norm_w),
-                                        ctypes.c_float(eps), _p(cs), _p(k_pool), _p(table), table.stride(0), _p(ctx.tok_seq),
+                                        ctypes.c_float(eps), _p(cs), _p(k_pool), _p(v_pool), _p(table), table.stride(0), _p(ctx.tok_seq),
                                         _p(ctx.tok_pos), T, n_heads, dim, rot, rot_dims, rank, hd, _stream()), "latent_prepare")
+
+
+LATENT_MFMA_MAX_ROW = 576
+
+
+def latent_attention_mfma(ctx, q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, table: torch.Tensor,
+                          n_heads: int, row: int, dv: int, scale: float, head_sink: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+    """bfloat16 attention over a latent cache on the matrix cores: q [T, heads, row], key rows and value rows
+    (the latent in the value pages' order) in pools [pages, 1, 64 * row]; returns [T, heads, dv], or None
+    for rows wider than the kernel takes.  Single-token steps share a sequence's pages out over several
+    blocks (chosen from the batch and the longest context the step may have) and merge."""
+    if q.dtype != torch.bfloat16 or row > LATENT_MFMA_MAX_ROW:
+        return None
+    T = ctx.n_tokens
+    _dev(q, k_pool, v_pool, table, head_sink, ctx.tok_pos, ctx.cu_dev)
+    _i32(table, "table")
+    _need(q.shape == (T, n_heads, row) and row % 16 == 0 and 0 < dv <= row, "latent attention: q must be [T, heads, row]")
+    _check_pools(k_pool, v_pool, 1, row, "latent attention")
+    _need(k_pool.dtype == torch.bfloat16 and v_pool is not None and v_pool.dtype == torch.bfloat16, "latent attention: bfloat16 pools")
+    if head_sink is not None:
+        _need(head_sink.dtype == torch.float32 and head_sink.shape == (n_heads,), "latent attention: head_sink must be float32 [heads]")
+    _need(table.dim() == 2 and table.shape[0] == ctx.batch, "latent attention: one table row a sequence")
+    lib = _lib()
+    splits, pps, ws, floats = 1, max(1, table.shape[1]), None, 0
+    if ctx.is_decode:
+        _need(T == ctx.batch, "latent attention: a single-token step has one token a sequence")
+        n_tiles = T * (-(-n_heads // 16))
+        pages = max(1, min(table.shape[1], -(-ctx.max_context // PAGE_TOKENS)))
+        want = max(1, (4 * compute_units()) // max(1, n_tiles))          # blocks of one wave's work: a few a compute unit
+        pps = max(1, -(-pages // min(pages, want)))
+        splits = -(-pages // pps)
+        cu = None
+        if splits > 1:
+            floats = lib.llogos_latent_attn_workspace(T * n_heads, dv, splits)
+            ws = _attn_workspace(q.device, floats)
+    else:
+        cu = ctx.cu_dev
+        _need(cu is not None and cu.numel() == ctx.batch + 1, "latent attention: the step's token offsets are missing")
+        n_tiles = sum(-(-(ctx.cu_seqlens[i + 1] - ctx.cu_seqlens[i]) * n_heads // 16) for i in range(ctx.batch))
+    out = torch.empty((T, n_heads, dv), dtype=torch.bfloat16, device=q.device)
+    code = lib.llogos_latent_attn_bf16(_p(out), dv, _p(q), _p(k_pool), _p(v_pool), _p(table), table.stride(0), _p(cu),
+                                       _p(ctx.tok_pos), ctx.batch, T, n_heads, row, ctypes.c_float(scale), _p(head_sink),
+                                       n_tiles, splits, pps, _p(ws), ctypes.c_longlong(ws.numel() if ws is not None else 0), _stream())
+    if code == -2:
+        return None
+    _check(code, "latent_attention_mfma")
+    return out
 
 
 def head_products(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:

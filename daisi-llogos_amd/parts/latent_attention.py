@@ -56,7 +56,11 @@ class LatentAttention(Mixer):
         return self.row
 
     def kv_spec(self) -> KVSpec:
-        return KVSpec(1, self.row, values=False)
+        # the matrix cores' attention (bfloat16, rows up to its limit) reads values in an operand order of their
+        # own: the latent is then cached a second time, as a value row; otherwise a value is part of its key row
+        rt = getattr(self, "rt", None)
+        mfma = rt is not None and rt.dtype == torch.bfloat16 and self.row <= K.LATENT_MFMA_MAX_ROW
+        return KVSpec(1, self.row, values=mfma)
 
     def tensor_specs(self) -> List[TensorSpec]:
         p, H = self.prefix, self.n_heads
@@ -95,12 +99,16 @@ class LatentAttention(Mixer):
         mark(ctx, "projections")
         cs = self.position.prepare(ctx) if self.position is not None else None
         qa = torch.empty((T, H, self.row), dtype=self.rt.dtype, device=h.device)
-        K.latent_prepare(ctx, kv, q, qa, self.c_norm_w, self.eps, cs, cache.k_pool, cache.table, H, self.dim, self.rot_dim,
+        K.latent_prepare(ctx, kv, q, qa, self.c_norm_w, self.eps, cs, cache.k_pool, cache.v_pool, cache.table, H, self.dim, self.rot_dim,
                          self.position.rot if self.position is not None else 0, self.kv_rank)
         K.head_products(q.view(T, H, self.dim + self.rot_dim)[:, :, :self.dim], self.uk_t, qa[:, :, :self.kv_rank])
         mark(ctx, "rotation")
-        lat = K.attention_generic(qa, H * self.row, cache.k_pool, None, cache.table, ctx.tok_seq, ctx.tok_pos, H, 1, self.row,
-                                  self.scale, v_dim=self.kv_rank, head_sink=self.sink)
+        lat = None
+        if cache.v_pool is not None:
+            lat = K.latent_attention_mfma(ctx, qa, cache.k_pool, cache.v_pool, cache.table, H, self.row, self.kv_rank, self.scale, self.sink)
+        if lat is None:
+            lat = K.attention_generic(qa, H * self.row, cache.k_pool, None, cache.table, ctx.tok_seq, ctx.tok_pos, H, 1, self.row,
+                                      self.scale, v_dim=self.kv_rank, head_sink=self.sink)
         mark(ctx, "attention")
         a = torch.empty((T, H, self.v_dim), dtype=self.rt.dtype, device=h.device)
         K.head_products(lat.view(T, H, self.kv_rank), self.uv, a)
