@@ -133,13 +133,30 @@ LLOGOS_EXPORT int llogos_token_shift(void* out, int out_dtype, const float* h, c
 // r, k, v, d, gate are float [T, H * D] (row stride ld); y is [T, H * D] in the output type.
 //
 // One block per (sequence, head).  Thread (j, part) keeps rows [part * rpt, (part + 1) * rpt) of
-// column j of S in registers; the P parts of a column are neighbouring lanes and add their
-// sums by shuffles, so the token loop needs no barrier.  Tokens go through LDS in chunks: a
-// chunk's r, k, w, v are loaded by all threads, its outputs are normed and stored by all
-// threads after the chunk's loop.  The state is stored [H][j][i] (a thread's rows in a row).
-// After its last token the block with head 0 copies the step's last mixer input row to the
-// sequence's `prev` state (the token-shift kernel has read the old one by then).
+// column j of S in registers; the P <= 16 parts of a column are neighbouring lanes of a row of 16 and add
+// their sums with cross-lane moves inside the vector unit, so the token loop needs no barrier and
+// no trip through LDS.  Few rows a thread (4 where a block of D * P threads allows) keep a token's
+// chain of dependent operations short: a long prompt of one sequence is a loop of as many steps as
+// it has tokens, on as many blocks as there are heads.  Tokens go through LDS in chunks: a chunk's
+// r, k, v, d, gate are asked for (into registers) while the chunk before is worked on, stored to LDS
+// (the decay made on the way), and the chunk's outputs are normed, gated and stored by all waves.
+// The state is stored [H][j][i] (a thread's rows in a row).  After its last token the block with
+// head 0 copies the step's last mixer input row to the sequence's `prev` state (the token-shift
+// kernel has read the old one by then).
 constexpr int kScanChunk = 16;
+constexpr int kScanAhead = 4;          // values of each array a thread asks for ahead (chunk <= kScanAhead * P tokens)
+
+__device__ __forceinline__ float dpp_add(float x, int ctrl_index) {
+    const int v = __float_as_int(x);
+    int o;
+    switch (ctrl_index) {
+        case 0: o = __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xf, 0xf, false); break;     // lane ^ 1 within a quad
+        case 1: o = __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xf, 0xf, false); break;     // lane ^ 2 within a quad
+        case 2: o = __builtin_amdgcn_update_dpp(0, v, 0x141, 0xf, 0xf, false); break;    // mirror within 8 lanes
+        default: o = __builtin_amdgcn_update_dpp(0, v, 0x140, 0xf, 0xf, false); break;   // mirror within 16 lanes
+    }
+    return x + __int_as_float(o);
+}
 
 template <int RPT, typename TO>
 __global__ void wkv_scan_kernel(TO* __restrict__ y, const float* __restrict__ r, const float* __restrict__ k,
@@ -149,7 +166,7 @@ __global__ void wkv_scan_kernel(TO* __restrict__ y, const float* __restrict__ r,
                                 float* __restrict__ state, size_t state_stride, size_t prev_offset,
                                 const float* __restrict__ h_in, int W,
                                 const int* __restrict__ slots, const int* __restrict__ cu,
-                                int H, int D, int P, int rpt) {
+                                int H, int D, int P, int rpt, int chunk) {
     extern __shared__ float smem[];
     const int seq = blockIdx.x, head = blockIdx.y;
     const int first = cu ? cu[seq] : seq, count = cu ? cu[seq + 1] - first : 1;
@@ -158,47 +175,87 @@ __global__ void wkv_scan_kernel(TO* __restrict__ y, const float* __restrict__ r,
     const bool active = j < D;
     const int i0 = part * rpt;
     float* s_r = smem;                          // [chunk][D]
-    float* s_k = s_r + kScanChunk * D;
-    float* s_w = s_k + kScanChunk * D;
-    float* s_v = s_w + kScanChunk * D;
-    float* s_o = s_v + kScanChunk * D;
-    float* s_u = s_o + kScanChunk * D;          // [D]
+    float* s_k = s_r + chunk * D;
+    float* s_w = s_k + chunk * D;
+    float* s_v = s_w + chunk * D;
+    float* s_g = s_v + chunk * D;
+    float* s_o = s_g + chunk * D;
     float* row = state + (size_t)slots[seq] * state_stride;
     float* S = row + ((size_t)head * D + (active ? j : 0)) * D + i0;
-
-    float s[RPT];
-#pragma unroll
-    for (int m = 0; m < RPT; ++m) s[m] = (active && m < rpt && i0 + m < D) ? S[m] : 0.f;
-    for (int i = tid; i < D; i += nthreads) s_u[i] = u[head * D + i];
-
     const size_t col0 = (size_t)head * D;
-    for (int c0 = 0; c0 < count; c0 += kScanChunk) {
-        const int n = min(kScanChunk, count - c0);
+
+    float s[RPT], ur[RPT];
+#pragma unroll
+    for (int m = 0; m < RPT; ++m) {
+        const bool ok = active && m < rpt && i0 + m < D;
+        s[m] = ok ? S[m] : 0.f;
+        ur[m] = ok ? u[col0 + i0 + m] : 0.f;
+    }
+    const bool vec = (rpt % 4 == 0) && (D % 4 == 0) && (i0 + rpt <= D);      // this thread's rows as float4 reads
+
+    // a chunk's values on their way: element e = tid + a * nthreads of the chunk's [n][D]
+    float pr[kScanAhead], pk[kScanAhead], pv[kScanAhead], pd[kScanAhead], pg[kScanAhead];
+    auto ask = [&](int c0) {
+        const int n = min(chunk, count - c0);
+#pragma unroll
+        for (int a = 0; a < kScanAhead; ++a) {
+            const int e = tid + a * nthreads;
+            if (e < n * D) {
+                const size_t at = (size_t)(first + c0 + e / D) * ld + col0 + e % D;
+                pr[a] = r[at]; pk[a] = k[at]; pv[a] = v[at]; pd[a] = d[at]; pg[a] = gate[at];
+            }
+        }
+    };
+    ask(0);
+    for (int c0 = 0; c0 < count; c0 += chunk) {
+        const int n = min(chunk, count - c0);
         __syncthreads();                        // the chunk before has been normed and stored
-        for (int e = tid; e < n * D; e += nthreads) {
-            const int c = e / D, i = e % D;
-            const size_t at = (size_t)(first + c0 + c) * ld + col0 + i;
-            s_r[e] = r[at];
-            s_k[e] = k[at];
-            s_v[e] = v[at];
-            s_w[e] = expf(-expf(d[at] + w0[col0 + i]));
+#pragma unroll
+        for (int a = 0; a < kScanAhead; ++a) {
+            const int e = tid + a * nthreads;
+            if (e < n * D) {
+                s_r[e] = pr[a]; s_k[e] = pk[a]; s_v[e] = pv[a]; s_g[e] = pg[a];
+                s_w[e] = expf(-expf(pd[a] + w0[col0 + e % D]));
+            }
         }
         __syncthreads();
+        if (c0 + chunk < count) ask(c0 + chunk);
         for (int c = 0; c < n; ++c) {
             const float* rr = s_r + c * D + i0;
             const float* kk = s_k + c * D + i0;
             const float* ww = s_w + c * D + i0;
             const float vj = active ? s_v[c * D + j] : 0.f;
             float acc = 0.f;
+            if (vec) {
 #pragma unroll
-            for (int m = 0; m < RPT; ++m) {
-                if (m < rpt && i0 + m < D) {
-                    const float kv = kk[m] * vj;
-                    acc = fmaf(rr[m], fmaf(s_u[i0 + m], kv, s[m]), acc);
-                    s[m] = fmaf(ww[m], s[m], kv);
+                for (int m = 0; m < RPT; m += 4) {
+                    if (m < rpt) {
+                        const float4 r4 = *reinterpret_cast<const float4*>(rr + m);
+                        const float4 k4 = *reinterpret_cast<const float4*>(kk + m);
+                        const float4 w4 = *reinterpret_cast<const float4*>(ww + m);
+                        const float rv[4] = {r4.x, r4.y, r4.z, r4.w}, kv4[4] = {k4.x, k4.y, k4.z, k4.w}, wv[4] = {w4.x, w4.y, w4.z, w4.w};
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            const float kv = kv4[q] * vj;
+                            acc = fmaf(rv[q], fmaf(ur[m + q], kv, s[m + q]), acc);
+                            s[m + q] = fmaf(wv[q], s[m + q], kv);
+                        }
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int m = 0; m < RPT; ++m) {
+                    if (m < rpt && i0 + m < D) {
+                        const float kv = kk[m] * vj;
+                        acc = fmaf(rr[m], fmaf(ur[m], kv, s[m]), acc);
+                        s[m] = fmaf(ww[m], s[m], kv);
+                    }
                 }
             }
-            for (int o = 1; o < P; o <<= 1) acc += __shfl_xor(acc, o, kWave);
+            if (P >= 2) acc = dpp_add(acc, 0);
+            if (P >= 4) acc = dpp_add(acc, 1);
+            if (P >= 8) acc = dpp_add(acc, 2);
+            if (P >= 16) acc = dpp_add(acc, 3);
             if (active && part == 0) s_o[c * D + j] = acc;
         }
         __syncthreads();
@@ -211,7 +268,7 @@ __global__ void wkv_scan_kernel(TO* __restrict__ y, const float* __restrict__ r,
             const float inv = 1.0f / sqrtf(ss / (float)D + eps);
             const size_t base = (size_t)(first + c0 + c);
             for (int i = lane; i < D; i += kWave) {
-                const float z = gate[base * ld + col0 + i];
+                const float z = s_g[c * D + i];
                 const float sg = z / (1.0f + expf(-z));
                 store_f32(y + base * (size_t)H * D + col0 + i, s_o[c * D + i] * inv * g[col0 + i] * sg);
             }
@@ -231,23 +288,81 @@ LLOGOS_EXPORT int llogos_wkv_scan(void* y, int out_dtype, const float* r, const 
                                   float* state, long long state_stride, long long prev_offset, const float* h_in, int W,
                                   const int* slots, const int* cu, int B, int H, int D, hipStream_t stream) {
     if (B <= 0 || H <= 0 || D <= 0 || ld < H * D) return LLOGOS_BAD_ARGUMENT;
-    if (D > 256) return LLOGOS_UNSUPPORTED;
-    // parts of a column: a power of two, rows a part <= 16 where the block then stays within 1024 threads
-    int rpt_max = 16, P = 1;
-    while (P * rpt_max < D) P <<= 1;
-    if ((long long)D * P > 1024) { rpt_max = 64; P = 1; while (P * rpt_max < D) P <<= 1; }
+    // rows a thread: the fewest of 4, 16, 64 with which a column's parts (a power of two, at most 16: one
+    // row of lanes) make a block of at most 1024 threads
+    int rpt_max = 0, P = 1;
+    for (int cand : {4, 16, 64}) {
+        P = 1;
+        while (P * cand < D) P <<= 1;
+        if (P <= 16 && (long long)((D * P + kWave - 1) / kWave * kWave) <= 1024) { rpt_max = cand; break; }
+    }
+    if (!rpt_max) return LLOGOS_UNSUPPORTED;
     const int rpt = (D + P - 1) / P;
-    int threads = D * P;
-    threads = (threads + kWave - 1) / kWave * kWave;
-    if (threads > 1024) return LLOGOS_UNSUPPORTED;
-    const size_t smem = (size_t)(5 * kScanChunk + 1) * D * sizeof(float);
+    const int threads = (D * P + kWave - 1) / kWave * kWave;
+    const int chunk = kScanChunk < kScanAhead * P ? kScanChunk : kScanAhead * P;     // so that a thread asks for <= kScanAhead values
+    const size_t smem = (size_t)6 * chunk * D * sizeof(float);
+    if (smem > 65536) return LLOGOS_UNSUPPORTED;
     dim3 grid(B, H);
 #define SCAN(RPT, TO) wkv_scan_kernel<RPT, TO><<<grid, threads, smem, stream>>>((TO*)y, r, k, v, d, gate, ld, w0, u, g, eps, \
-        state, (size_t)state_stride, (size_t)prev_offset, h_in, W, slots, cu, H, D, P, rpt)
-    if (out_dtype == DT_F32) { if (rpt_max == 16) SCAN(16, float); else SCAN(64, float); }
-    else if (out_dtype == DT_BF16) { if (rpt_max == 16) SCAN(16, bf16_t); else SCAN(64, bf16_t); }
+        state, (size_t)state_stride, (size_t)prev_offset, h_in, W, slots, cu, H, D, P, rpt, chunk)
+#define SCANS(TO) do { if (rpt_max == 4) SCAN(4, TO); else if (rpt_max == 16) SCAN(16, TO); else SCAN(64, TO); } while (0)
+    if (out_dtype == DT_F32) SCANS(float);
+    else if (out_dtype == DT_BF16) SCANS(bf16_t);
     else return LLOGOS_BAD_ARGUMENT;
+#undef SCANS
 #undef SCAN
+    return LLOGOS_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------- a norm after a sublayer, the sum, the next norm
+// For a block with norms on both sides of its sublayers:  x += norm_b(a) and then h = norm_n(x), one
+// block a row, the row in LDS between the two passes:
+//     v = sum of the parts of a;   x <- x + v / sqrt(mean(v^2) + eps) * wb
+//     h = x / sqrt(mean(x^2) + eps) * wn           (skipped without wn)
+// x is the float residual stream (written back), a the sublayer's output (float or bfloat16,
+// maybe in parts of a k-split product), h the rows the next sublayer reads.
+template <typename TA, typename TH>
+__global__ void sandwich_norm_kernel(float* __restrict__ x, const TA* __restrict__ a, int parts, size_t part_stride,
+                                     const float* __restrict__ wb, const float* __restrict__ wn, TH* __restrict__ h,
+                                     float eps, int H) {
+    extern __shared__ float rowbuf[];
+    __shared__ float red[16];
+    const size_t r = blockIdx.x;
+    float* xr = x + r * H;
+    const TA* ar = a + r * H;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+        float v = load_f32(ar + i);
+        for (int q = 1; q < parts; ++q) v += load_f32(ar + q * part_stride + i);
+        rowbuf[i] = v;
+        ss = fmaf(v, v, ss);
+    }
+    const float inv_a = 1.0f / sqrtf(block_sum(ss, red) / (float)H + eps);
+    ss = 0.f;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+        const float v = fmaf(rowbuf[i] * inv_a, wb[i], xr[i]);
+        xr[i] = v;
+        rowbuf[i] = v;
+        ss = fmaf(v, v, ss);
+    }
+    if (!wn) return;
+    const float inv_x = 1.0f / sqrtf(block_sum(ss, red) / (float)H + eps);
+    TH* hr = h + r * H;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) store_f32(hr + i, rowbuf[i] * inv_x * wn[i]);
+}
+
+LLOGOS_EXPORT int llogos_sandwich_norm(float* x, const void* a, int a_dtype, int parts, long long part_stride, const float* wb,
+                                       const float* wn, void* h, int h_dtype, float eps, int T, int H, hipStream_t stream) {
+    if (T <= 0 || H <= 0 || parts < 1 || (size_t)H * sizeof(float) > 65536) return LLOGOS_BAD_ARGUMENT;
+    const int threads = H >= 2048 ? 512 : (H >= 512 ? 256 : 128);
+    const size_t smem = (size_t)H * sizeof(float);
+#define SN(TA, TH) sandwich_norm_kernel<TA, TH><<<T, threads, smem, stream>>>(x, (const TA*)a, parts, (size_t)part_stride, wb, wn, (TH*)h, eps, H)
+    if (a_dtype == DT_F32 && h_dtype == DT_F32) SN(float, float);
+    else if (a_dtype == DT_F32 && h_dtype == DT_BF16) SN(float, bf16_t);
+    else if (a_dtype == DT_BF16 && h_dtype == DT_F32) SN(bf16_t, float);
+    else if (a_dtype == DT_BF16 && h_dtype == DT_BF16) SN(bf16_t, bf16_t);
+    else return LLOGOS_BAD_ARGUMENT;
+#undef SN
     return LLOGOS_LAUNCH_CHECK();
 }
 

@@ -234,6 +234,9 @@ def qk_rope_cache(qkv: torch.Tensor, bias: Optional[torch.Tensor], out_dtype: to
     return q_out
 
 
+GENERIC_MAX_HEAD_DIM = 1024      # the widest row the kernel for any shape takes (kMaxHeadDimGeneric)
+
+
 def attention_generic(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torch.Tensor,
                       table: torch.Tensor, tok_seq: torch.Tensor, tok_pos: torch.Tensor,
                       n_heads: int, n_kv_heads: int, head_dim: int, scale: float,
@@ -248,7 +251,7 @@ def attention_generic(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_po
     T = tok_seq.numel()
     _need(q.is_cuda and q.dtype == k_pool.dtype, "attention: q and cache types differ")
     _need(n_heads % n_kv_heads == 0, "attention: heads must be a multiple of kv heads")
-    _need(0 < head_dim <= MAX_HEAD_DIM, f"attention: head_dim {head_dim} not in 1..{MAX_HEAD_DIM}")
+    _need(0 < head_dim <= GENERIC_MAX_HEAD_DIM, f"attention: head_dim {head_dim} not in 1..{GENERIC_MAX_HEAD_DIM}")
     _check_pools(k_pool, v_pool, n_kv_heads, head_dim, "attention")
     _need(q_stride >= n_heads * head_dim and q.numel() >= (T - 1) * q_stride + n_heads * head_dim,
           "attention: q too small")
@@ -367,12 +370,31 @@ def wkv_scan(ctx, r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, d: torch.Te
     _need(h_in.dtype == torch.float32 and h_in.shape == (ctx.n_tokens, W), "wkv_scan: h_in must be float32 [T, W]")
     _need(state.dtype == torch.float32 and state.dim() == 2 and state.shape[1] == HD * dim + W, "wkv_scan: state must be float32 [slots, heads * dim * dim + W]")
     _need(ctx.cu_dev is not None or ctx.n_tokens == ctx.batch, "wkv_scan: a step of several tokens a sequence needs the token offsets")
-    _need((5 * 16 + 1) * dim * 4 <= 65536, f"wkv_scan: head size {dim} is too large")
+    _need(6 * 16 * dim * 4 <= 65536, f"wkv_scan: head size {dim} is too large")
     y = torch.empty((ctx.n_tokens, HD), dtype=out_dtype, device=r.device)
     _check(_lib().llogos_wkv_scan(_p(y), _DT[out_dtype], _p(r), _p(k), _p(v), _p(d), _p(gate), HD, _p(w0), _p(u), _p(g),
                                   ctypes.c_float(eps), _p(state), ctypes.c_longlong(state.stride(0)), ctypes.c_longlong(HD * dim),
                                   _p(h_in), W, _p(ctx.slots), _p(ctx.cu_dev), ctx.batch, n_heads, dim, _stream()), "wkv_scan")
     return y
+
+
+def sandwich_norm(x: torch.Tensor, a: torch.Tensor, post_w: torch.Tensor, next_w: Optional[torch.Tensor], eps: float,
+                  out_dtype: torch.dtype) -> Optional[torch.Tensor]:
+    """x += rmsnorm(a) * post_w in place (x the float32 stream [T, H]; a [T, H] or float32 partial sums
+    [parts, T, H]), and, with next_w, the rows rmsnorm(x) * next_w of the completed stream in `out_dtype`."""
+    _dev(x, a, post_w, next_w)
+    _need(x.dtype == torch.float32 and x.dim() == 2, "sandwich_norm: x must be float32 [T, H]")
+    T, H = x.shape
+    parts, part_stride = _parts(a)
+    _need(tuple(a.shape[-2:]) == (T, H) and (parts == 1 or a.dtype == torch.float32), "sandwich_norm: a must have x's shape")
+    _need(post_w.dtype == torch.float32 and post_w.shape == (H,), "sandwich_norm: weights must be float32 [H]")
+    _need(next_w is None or (next_w.dtype == torch.float32 and next_w.shape == (H,)), "sandwich_norm: weights must be float32 [H]")
+    _need(H * 4 <= 65536, "sandwich_norm: rows of more than 16,384 values")
+    h = torch.empty((T, H), dtype=out_dtype, device=x.device) if next_w is not None else None
+    if T:
+        _check(_lib().llogos_sandwich_norm(_p(x), _p(a), _dt(a), parts, ctypes.c_longlong(part_stride), _p(post_w), _p(next_w),
+                                           _p(h), _DT[out_dtype], ctypes.c_float(eps), T, H, _stream()), "sandwich_norm")
+    return h
 
 
 def activation(x: torch.Tensor, kind: str, out_dtype: torch.dtype, a: float = 0.0, b: float = 0.0) -> torch.Tensor:

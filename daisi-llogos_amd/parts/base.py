@@ -176,6 +176,15 @@ class NormedRows:
         return self.norm.forward(self.x)
 
 
+@dataclass
+class NormedAhead:
+    """What a block hands on instead of a delta when it has completed the stream itself and already made
+    the rows that `norm` would make of it (float32, all rows): the norm named here returns them when it is
+    asked for just that, and any other norm, or a request for some rows or another type, norms the stream."""
+    rows: torch.Tensor
+    norm: "Norm"
+
+
 class Mixer(Part):
     """Token mixer: forward(ctx, h [T, H] in the runtime's type, cache) -> [T, H], or float32
     partial sums [parts, T, H] that the residual sum after it adds.

@@ -13,7 +13,8 @@ from typing import Callable, List, Optional, Tuple
 
 import torch
 
-from .base import Block, FeedForward, LayerCache, Mixer, Norm, Part, Residual, Runtime, StepContext, TensorSpec, mark, register_block
+from .base import Block, FeedForward, LayerCache, Mixer, Norm, NormedAhead, Part, Residual, Runtime, StepContext, TensorSpec, mark, register_block
+from .norm import RMSNorm
 
 
 @register_block("pre_norm")
@@ -100,6 +101,8 @@ class SandwichBlock(Block):
     def entry_norm(self) -> Optional[Norm]:
         return self.mixer_norm
 
+    takes_next_norm = True
+
     def _read(self, ctx, norm: Norm, conv, x, delta, cache, want_f32: bool):
         """What a sublayer reads: norm(x + delta), through the convolution when there is one."""
         dtype = torch.float32 if want_f32 else self.rt.dtype
@@ -109,31 +112,45 @@ class SandwichBlock(Block):
         mark(ctx, "norm")
         return conv.forward(ctx, h, cache, out_dtype=dtype)
 
-    @staticmethod
-    def _float_rows(out: torch.Tensor) -> torch.Tensor:
-        """A part's output as one float32 [T, H] tensor (a norm's input)."""
-        if out.dim() == 2 and out.dtype == torch.float32:
-            return out
+    def _close(self, x, out, post: Norm, nxt: Optional[Norm], rows_f32: bool):
+        """A sublayer's output `out` joins the stream through its norm `post`, and the norm `nxt` that
+        reads the stream next is applied on the way: one kernel for both where both are RMS norms over the
+        stream's width (then x is complete and the rows are returned), else the norm's own kernel (then the
+        normed output is returned as a delta that the next norm adds).  Returns (rows or None, delta or None).
+        The rows handed to another block are float32 (a convolution or a mixer that mixes rows reads them)."""
         from ..ops import kernels as K
-        return K.sum_parts(out, None, torch.float32)
+        fused = isinstance(post, RMSNorm) and (nxt is None or isinstance(nxt, RMSNorm)) and x.shape[1] * 4 <= 65536 \
+            and (nxt is None or nxt.eps == post.eps)
+        if not fused:
+            a = out if (out.dim() == 2 and out.dtype == torch.float32) else K.sum_parts(out, None, torch.float32)
+            return None, post.forward(a, out_dtype=torch.float32)
+        dtype = torch.float32 if rows_f32 else self.rt.dtype
+        rows = K.sandwich_norm(x, out, post.weight, nxt.weight if nxt is not None else None, post.eps, dtype)
+        return rows, None
 
-    def forward(self, ctx: StepContext, x: torch.Tensor, pending, caches):
+    def forward(self, ctx: StepContext, x: torch.Tensor, pending, caches, next_norm: Optional[Norm] = None):
         caches = list(caches)
         conv1_cache = caches.pop(0) if self.mixer_conv is not None else None
         mixer_cache = caches.pop(0)
         conv2_cache = caches.pop(0) if self.ffn_conv is not None else None
-        h = self._read(ctx, self.mixer_norm, self.mixer_conv, x, pending, conv1_cache, self.mixer.takes_float32_rows)
+        f32_in = self.mixer.takes_float32_rows
+        h = self._read(ctx, self.mixer_norm, self.mixer_conv, x, pending, conv1_cache, f32_in)
         mark(ctx, "conv" if self.mixer_conv is not None else "norm")
-        a = self._float_rows(self.mixer.forward(ctx, h, mixer_cache))
+        a = self.mixer.forward(ctx, h, mixer_cache)
         mark(ctx, "mixer")
-        delta = self.post_mixer_norm.forward(a, out_dtype=torch.float32)
-        mark(ctx, "norm")
         if self.ffn is None:
-            return x, delta
-        h = self._read(ctx, self.ffn_norm, self.ffn_conv, x, delta, conv2_cache, False)
-        mark(ctx, "conv" if self.ffn_conv is not None else "norm")
-        d = self._float_rows(self.ffn.forward(ctx, h))
-        mark(ctx, "feed_forward")
-        delta = self.post_ffn_norm.forward(d, out_dtype=torch.float32)
+            rows, delta = self._close(x, a, self.post_mixer_norm, next_norm, True)
+            mark(ctx, "norm")
+            return x, (delta if rows is None else NormedAhead(rows, next_norm))
+        rows, delta = self._close(x, a, self.post_mixer_norm, self.ffn_norm, self.ffn_conv is not None)
         mark(ctx, "norm")
-        return x, delta
+        if rows is None:
+            h = self._read(ctx, self.ffn_norm, self.ffn_conv, x, delta, conv2_cache, False)
+        else:
+            h = self.ffn_conv.forward(ctx, rows, conv2_cache, out_dtype=self.rt.dtype) if self.ffn_conv is not None else rows
+        mark(ctx, "conv" if self.ffn_conv is not None else "norm")
+        d = self.ffn.forward(ctx, h)
+        mark(ctx, "feed_forward")
+        rows, delta = self._close(x, d, self.post_ffn_norm, next_norm, True)
+        mark(ctx, "norm")
+        return x, (delta if rows is None else NormedAhead(rows, next_norm))

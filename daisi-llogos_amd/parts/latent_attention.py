@@ -92,10 +92,11 @@ class LatentAttention(Mixer):
 
     def forward(self, ctx: StepContext, h: torch.Tensor, cache: LayerCache) -> torch.Tensor:
         f32, H, T = torch.float32, self.n_heads, ctx.n_tokens
-        cq = self.dq.forward(h, out_dtype=f32)
+        plain = lambda p: K.sum_parts(p, None, f32)          # (a product may come as partial sums of a split along k)
+        cq = plain(self.dq.product(h, f32_ok=True))
         cq = K.rmsnorm(cq, self.q_norm_w, self.eps, self.rt.dtype)
-        q = self.uq.forward(cq, out_dtype=f32)                                   # [T, H * (dim + rot)]
-        kv = self.dkv.forward(h, out_dtype=f32)                                  # [T, rank + rot]
+        q = plain(self.uq.product(cq, f32_ok=True))                               # [T, H * (dim + rot)]
+        kv = plain(self.dkv.product(h, f32_ok=True))                              # [T, rank + rot]
         mark(ctx, "projections")
         cs = self.position.prepare(ctx) if self.position is not None else None
         qa = torch.empty((T, H, self.row), dtype=self.rt.dtype, device=h.device)
@@ -112,6 +113,6 @@ class LatentAttention(Mixer):
         mark(ctx, "attention")
         a = torch.empty((T, H, self.v_dim), dtype=self.rt.dtype, device=h.device)
         K.head_products(lat.view(T, H, self.kv_rank), self.uv, a)
-        out = self.o.forward(a.view(T, H * self.v_dim), out_dtype=f32)
+        out = self.o.product(a.view(T, H * self.v_dim), f32_ok=True)
         mark(ctx, "o")
         return out

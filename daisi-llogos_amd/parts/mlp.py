@@ -92,6 +92,6 @@ class ActivatedMLP(FeedForward):
         z = self.up.product(h, f32_ok=True)
         mark(ctx, "up")
         act = K.activation(z, self.activation, self.rt.dtype, self.a, self.b)
-        out = self.down.forward(act, out_dtype=torch.float32)
+        out = self.down.product(act, f32_ok=True)
         mark(ctx, "down")
         return out

@@ -9,7 +9,7 @@ from typing import Callable, List, Optional
 import torch
 
 from ..ops import kernels as K
-from .base import Norm, NormedRows, Runtime, TensorSpec, register_norm
+from .base import Norm, NormedAhead, NormedRows, Runtime, TensorSpec, register_norm
 
 
 @register_norm("rmsnorm")
@@ -38,6 +38,12 @@ class RMSNorm(Norm):
 
     def forward(self, x: torch.Tensor, delta=None, rows: Optional[torch.Tensor] = None,
                 write_back: bool = True, lazy: bool = False, out_dtype: Optional[torch.dtype] = None):
+        if isinstance(delta, NormedAhead):
+            # the block before has completed the stream and made this norm's rows on the way
+            want = out_dtype or self.rt.dtype
+            if delta.norm is self and rows is None and delta.rows.dtype == want:
+                return delta.rows
+            delta = None
         if isinstance(delta, K.RowSquares):
             # the product before has added itself to x; if it also left this norm's rows without their
             # scale, a consumer that takes them needs no kernel here

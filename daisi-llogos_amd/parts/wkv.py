@@ -71,13 +71,15 @@ class WKV(Mixer):
         prev = state[:, self.inner * self.head_dim:]
         m = K.token_shift(ctx, h, self.mu, prev, self.rt.dtype)                # [5, T, hidden]
         mark(ctx, "shift")
-        r, k, v, g = (lin.forward(m[i], out_dtype=f32) for i, lin in enumerate((self.r, self.k, self.v, self.g)))
-        low = K.activation(self.w1.forward(m[4], out_dtype=f32), "tanh", self.rt.dtype)
-        d = self.w2.forward(low, out_dtype=f32)
+        # (a product may come as float32 partial sums of a split along k: the activation adds them itself)
+        plain = lambda p: K.sum_parts(p, None, f32)
+        r, k, v, g = (plain(lin.product(m[i], f32_ok=True)) for i, lin in enumerate((self.r, self.k, self.v, self.g)))
+        low = K.activation(self.w1.product(m[4], f32_ok=True), "tanh", self.rt.dtype)
+        d = plain(self.w2.product(low, f32_ok=True))
         mark(ctx, "projections")
         y = K.wkv_scan(ctx, r, k, v, d, g, self.w0, self.u, self.norm_w, self.eps, state, self.n_heads, self.head_dim,
                        h, self.rt.dtype)
         mark(ctx, "recurrence")
-        out = self.o.forward(y, out_dtype=f32)
+        out = self.o.product(y, f32_ok=True)          # maybe in parts: the norm that follows adds them
         mark(ctx, "o")
         return out
