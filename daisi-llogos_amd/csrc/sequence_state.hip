@@ -130,7 +130,8 @@ LLOGOS_EXPORT int llogos_token_shift(void* out, int out_dtype, const float* h, c
 //     o_t[j] = sum_i r_t[i] * (S[i, j] + u[i] * k_t[i] * v_t[j])
 //     S[i, j] <- w_t[i] * S[i, j] + k_t[i] * v_t[j],      w_t[i] = exp(-exp(d_t[i] + w0[i]))
 // then y_t = o_t / sqrt(mean_j(o_t^2) + eps) * g[j] * silu(gate_t[j]) over the head's D channels.
-// r, k, v, d, gate are float [T, H * D] (row stride ld); y is [T, H * D] in the output type.
+// r, k, v, d, gate are float [T, H * D] (row stride ld), r, k, v, gate maybe as `parts` partial sums
+// (part_stride floats apart) and d as d_parts; y is [T, H * D] in the output type.
 //
 // One block per (sequence, head).  Thread (j, part) keeps rows [part * rpt, (part + 1) * rpt) of
 // column j of S in registers; the P <= 16 parts of a column are neighbouring lanes of a row of 16 and add
@@ -158,21 +159,27 @@ __device__ __forceinline__ float dpp_add(float x, int ctrl_index) {
     return x + __int_as_float(o);
 }
 
-template <int RPT, typename TO>
+// PP: parts of a column (a power of two up to 16); EXACT: every thread has exactly RPT rows (D = PP * RPT), read
+// as float4s without a bound check.  Both are template arguments so that a token's loop has no branch.
+template <int RPT, int PP, bool EXACT, typename TO>
 __global__ void wkv_scan_kernel(TO* __restrict__ y, const float* __restrict__ r, const float* __restrict__ k,
                                 const float* __restrict__ v, const float* __restrict__ d, const float* __restrict__ gate,
-                                int ld, const float* __restrict__ w0, const float* __restrict__ u,
+                                int ld, int parts, size_t part_stride, int d_parts, size_t d_part_stride,
+                                const float* __restrict__ w0, const float* __restrict__ u,
                                 const float* __restrict__ g, float eps,
                                 float* __restrict__ state, size_t state_stride, size_t prev_offset,
                                 const float* __restrict__ h_in, int W,
                                 const int* __restrict__ slots, const int* __restrict__ cu,
-                                int H, int D, int P, int rpt, int chunk) {
+                                int H, int D, int rpt, int chunk, int Dc, float* __restrict__ o_raw) {
+    constexpr int P = PP;
     extern __shared__ float smem[];
     const int seq = blockIdx.x, head = blockIdx.y;
     const int first = cu ? cu[seq] : seq, count = cu ? cu[seq + 1] - first : 1;
     const int tid = threadIdx.x, nthreads = blockDim.x;
-    const int j = tid / P, part = tid % P;
-    const bool active = j < D;
+    // the block's columns of S: all D, or, with several blocks a head (long prompts of few sequences: a
+    // compute unit issues a token's instructions for all of a block's waves), Dc of them from blockIdx.z * Dc on
+    const int j = blockIdx.z * Dc + tid / P, part = tid % P;
+    const bool active = tid / P < Dc && j < D;
     const int i0 = part * rpt;
     float* s_r = smem;                          // [chunk][D]
     float* s_k = s_r + chunk * D;
@@ -191,7 +198,6 @@ __global__ void wkv_scan_kernel(TO* __restrict__ y, const float* __restrict__ r,
         s[m] = ok ? S[m] : 0.f;
         ur[m] = ok ? u[col0 + i0 + m] : 0.f;
     }
-    const bool vec = (rpt % 4 == 0) && (D % 4 == 0) && (i0 + rpt <= D);      // this thread's rows as float4 reads
 
     // a chunk's values on their way: element e = tid + a * nthreads of the chunk's [n][D]
     float pr[kScanAhead], pk[kScanAhead], pv[kScanAhead], pd[kScanAhead], pg[kScanAhead];
@@ -202,7 +208,13 @@ __global__ void wkv_scan_kernel(TO* __restrict__ y, const float* __restrict__ r,
             const int e = tid + a * nthreads;
             if (e < n * D) {
                 const size_t at = (size_t)(first + c0 + e / D) * ld + col0 + e % D;
-                pr[a] = r[at]; pk[a] = k[at]; pv[a] = v[at]; pd[a] = d[at]; pg[a] = gate[at];
+                float xr = r[at], xk = k[at], xv = v[at], xd = d[at], xg = gate[at];
+                for (int q = 1; q < parts; ++q) {            // products that come as partial sums of a split along k
+                    xr += r[q * part_stride + at]; xk += k[q * part_stride + at];
+                    xv += v[q * part_stride + at]; xg += gate[q * part_stride + at];
+                }
+                for (int q = 1; q < d_parts; ++q) xd += d[q * d_part_stride + at];
+                pr[a] = xr; pk[a] = xk; pv[a] = xv; pd[a] = xd; pg[a] = xg;
             }
         }
     };
@@ -221,18 +233,20 @@ __global__ void wkv_scan_kernel(TO* __restrict__ y, const float* __restrict__ r,
         __syncthreads();
         if (c0 + chunk < count) ask(c0 + chunk);
         for (int c = 0; c < n; ++c) {
-            const float* rr = s_r + c * D + i0;
-            const float* kk = s_k + c * D + i0;
-            const float* ww = s_w + c * D + i0;
-            const float vj = active ? s_v[c * D + j] : 0.f;
+            // (indices into the one LDS array, so that every read is an LDS read whatever the optimizer infers)
+            const int at = c * D + i0, o_k = chunk * D, o_w = 2 * chunk * D;
+            const float* rr = smem + at;
+            const float* kk = smem + o_k + at;
+            const float* ww = smem + o_w + at;
+            const float vj = active ? smem[3 * chunk * D + c * D + j] : 0.f;
             float acc = 0.f;
-            if (vec) {
+            if (EXACT) {
 #pragma unroll
                 for (int m = 0; m < RPT; m += 4) {
-                    if (m < rpt) {
-                        const float4 r4 = *reinterpret_cast<const float4*>(rr + m);
-                        const float4 k4 = *reinterpret_cast<const float4*>(kk + m);
-                        const float4 w4 = *reinterpret_cast<const float4*>(ww + m);
+                    {
+                        const float4 r4 = *reinterpret_cast<const float4*>(&smem[at + m]);
+                        const float4 k4 = *reinterpret_cast<const float4*>(&smem[o_k + at + m]);
+                        const float4 w4 = *reinterpret_cast<const float4*>(&smem[o_w + at + m]);
                         const float rv[4] = {r4.x, r4.y, r4.z, r4.w}, kv4[4] = {k4.x, k4.y, k4.z, k4.w}, wv[4] = {w4.x, w4.y, w4.z, w4.w};
 #pragma unroll
                         for (int q = 0; q < 4; ++q) {
@@ -256,9 +270,17 @@ __global__ void wkv_scan_kernel(TO* __restrict__ y, const float* __restrict__ r,
             if (P >= 4) acc = dpp_add(acc, 1);
             if (P >= 8) acc = dpp_add(acc, 2);
             if (P >= 16) acc = dpp_add(acc, 3);
-            if (active && part == 0) s_o[c * D + j] = acc;
+            if (active && part == 0) smem[5 * chunk * D + c * D + j] = acc;
         }
         __syncthreads();
+        if (o_raw) {
+            // several blocks a head: the raw outputs of this block's columns; head_norm_gate_kernel norms the head
+            for (int e = tid; e < n * Dc; e += nthreads) {
+                const int c = e / Dc, jj = blockIdx.z * Dc + e % Dc;
+                if (jj < D) o_raw[(size_t)(first + c0 + c) * H * D + col0 + jj] = s_o[c * D + jj];
+            }
+            continue;
+        }
         // norm over the head, weight, gate: a wave takes a token at a time
         const int wave = tid / kWave, lane = tid % kWave, nwaves = (nthreads + kWave - 1) / kWave;
         for (int c = wave; c < n; c += nwaves) {
@@ -277,17 +299,40 @@ __global__ void wkv_scan_kernel(TO* __restrict__ y, const float* __restrict__ r,
 #pragma unroll
     for (int m = 0; m < RPT; ++m)
         if (active && m < rpt && i0 + m < D) S[m] = s[m];
-    if (head == 0 && h_in) {
+    if (head == 0 && blockIdx.z == 0 && h_in) {
         const float* last = h_in + (size_t)(first + count - 1) * W;
         for (int c = tid; c < W; c += nthreads) row[prev_offset + c] = last[c];
     }
 }
 
+// y[t, head, :] = o / sqrt(mean(o^2) + eps) * g * silu(gate) over each head's D channels; one wave a (token, head).
+template <typename TO>
+__global__ void head_norm_gate_kernel(TO* __restrict__ y, const float* __restrict__ o, const float* __restrict__ gate, int ld,
+                                      int parts, size_t part_stride, const float* __restrict__ g, float eps, int H, int D, int n) {
+    const int item = blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    if (item >= n) return;
+    const int t = item / H, head = item % H;
+    const float* orow = o + (size_t)t * H * D + (size_t)head * D;
+    float ss = 0.f;
+    for (int i = lane; i < D; i += kWave) ss = fmaf(orow[i], orow[i], ss);
+    ss = wave_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / (float)D + eps);
+    for (int i = lane; i < D; i += kWave) {
+        float z = gate[(size_t)t * ld + (size_t)head * D + i];
+        for (int q = 1; q < parts; ++q) z += gate[q * part_stride + (size_t)t * ld + (size_t)head * D + i];
+        store_f32(y + (size_t)t * H * D + (size_t)head * D + i, orow[i] * inv * g[head * D + i] * (z / (1.0f + expf(-z))));
+    }
+}
+
+// col_blocks > 1 (with o_raw, float [T, H * D] scratch): a head's columns are shared out over that many blocks
+// and the head norm runs as a second kernel.
 LLOGOS_EXPORT int llogos_wkv_scan(void* y, int out_dtype, const float* r, const float* k, const float* v, const float* d,
-                                  const float* gate, int ld, const float* w0, const float* u, const float* g, float eps,
+                                  const float* gate, int ld, int parts, long long part_stride, int d_parts,
+                                  long long d_part_stride, const float* w0, const float* u, const float* g, float eps,
                                   float* state, long long state_stride, long long prev_offset, const float* h_in, int W,
-                                  const int* slots, const int* cu, int B, int H, int D, hipStream_t stream) {
-    if (B <= 0 || H <= 0 || D <= 0 || ld < H * D) return LLOGOS_BAD_ARGUMENT;
+                                  const int* slots, const int* cu, int B, int H, int D, int T, int col_blocks, float* o_raw,
+                                  hipStream_t stream) {
+    if (B <= 0 || H <= 0 || D <= 0 || ld < H * D || parts < 1 || d_parts < 1 || col_blocks < 1 || (col_blocks > 1 && !o_raw)) return LLOGOS_BAD_ARGUMENT;
     // rows a thread: the fewest of 4, 16, 64 with which a column's parts (a power of two, at most 16: one
     // row of lanes) make a block of at most 1024 threads
     int rpt_max = 0, P = 1;
@@ -298,19 +343,40 @@ LLOGOS_EXPORT int llogos_wkv_scan(void* y, int out_dtype, const float* r, const 
     }
     if (!rpt_max) return LLOGOS_UNSUPPORTED;
     const int rpt = (D + P - 1) / P;
-    const int threads = (D * P + kWave - 1) / kWave * kWave;
-    const int chunk = kScanChunk < kScanAhead * P ? kScanChunk : kScanAhead * P;     // so that a thread asks for <= kScanAhead values
+    const int Dc = (D + col_blocks - 1) / col_blocks;
+    const int threads = (Dc * P + kWave - 1) / kWave * kWave;
+    // so that a thread asks for <= kScanAhead values of a chunk's [tokens][D]
+    int chunk = kScanChunk;
+    while (chunk > 1 && (long long)chunk * D > (long long)kScanAhead * threads) chunk >>= 1;
+    if ((long long)chunk * D > (long long)kScanAhead * threads) return LLOGOS_UNSUPPORTED;
+    while (chunk > 1 && (size_t)6 * chunk * D * sizeof(float) > 65536) chunk >>= 1;
     const size_t smem = (size_t)6 * chunk * D * sizeof(float);
     if (smem > 65536) return LLOGOS_UNSUPPORTED;
-    dim3 grid(B, H);
-#define SCAN(RPT, TO) wkv_scan_kernel<RPT, TO><<<grid, threads, smem, stream>>>((TO*)y, r, k, v, d, gate, ld, w0, u, g, eps, \
-        state, (size_t)state_stride, (size_t)prev_offset, h_in, W, slots, cu, H, D, P, rpt, chunk)
-#define SCANS(TO) do { if (rpt_max == 4) SCAN(4, TO); else if (rpt_max == 16) SCAN(16, TO); else SCAN(64, TO); } while (0)
+    if (col_blocks == 1) o_raw = nullptr;
+    dim3 grid(B, H, col_blocks);
+#define ARGS(TO) ((TO*)y, r, k, v, d, gate, ld, parts, (size_t)part_stride, d_parts, (size_t)d_part_stride, w0, u, g, eps, \
+        state, (size_t)state_stride, (size_t)prev_offset, h_in, W, slots, cu, H, D, rpt, chunk, Dc, o_raw)
+    const bool exact = rpt == rpt_max && P * rpt == D;
+#define SCAN(RPT, PP, TO) do { if (exact) wkv_scan_kernel<RPT, PP, true, TO><<<grid, threads, smem, stream>>> ARGS(TO); \
+                               else wkv_scan_kernel<RPT, PP, false, TO><<<grid, threads, smem, stream>>> ARGS(TO); } while (0)
+#define SCANS(TO) do { \
+        if (rpt_max == 4) { if (P == 1) SCAN(4, 1, TO); else if (P == 2) SCAN(4, 2, TO); else if (P == 4) SCAN(4, 4, TO); \
+                            else if (P == 8) SCAN(4, 8, TO); else SCAN(4, 16, TO); } \
+        else if (rpt_max == 16) { if (P == 8) SCAN(16, 8, TO); else SCAN(16, 16, TO); } \
+        else { if (P == 4) SCAN(64, 4, TO); else return LLOGOS_UNSUPPORTED; } } while (0)
     if (out_dtype == DT_F32) SCANS(float);
     else if (out_dtype == DT_BF16) SCANS(bf16_t);
     else return LLOGOS_BAD_ARGUMENT;
 #undef SCANS
 #undef SCAN
+#undef ARGS
+    if (o_raw) {
+        const int n = T * H, waves = 4;
+        if (out_dtype == DT_F32)
+            head_norm_gate_kernel<float><<<(n + waves - 1) / waves, waves * kWave, 0, stream>>>((float*)y, o_raw, gate, ld, parts, (size_t)part_stride, g, eps, H, D, n);
+        else
+            head_norm_gate_kernel<bf16_t><<<(n + waves - 1) / waves, waves * kWave, 0, stream>>>((bf16_t*)y, o_raw, gate, ld, parts, (size_t)part_stride, g, eps, H, D, n);
+    }
     return LLOGOS_LAUNCH_CHECK();
 }
 

@@ -74,6 +74,10 @@ def main(argv=None) -> int:
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens live requests hold at any time (each rounded up to 64); sizes the cache")
     args = ap.parse_args(argv)
-    engine = Engine.from_folder(args.model, dtype=args.dtype, max_tokens=args.max_tokens)
+    # a request holds whole pages: one page more for each of the slots the engine starts with covers every
+    # request's last, partly filled page whatever way the caller counted
+    from ..cache.pages import PAGE_TOKENS
+    n_slots = 64
+    engine = Engine.from_folder(args.model, dtype=args.dtype, max_tokens=args.max_tokens + n_slots * PAGE_TOKENS, n_slots=n_slots)
     replay(engine, sys.stdin, args.out)
     return 0

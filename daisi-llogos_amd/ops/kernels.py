@@ -357,25 +357,55 @@ def wkv_scan(ctx, r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, d: torch.Te
              dim: int, h_in: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
     """The recurrence S <- diag(w) S + k v^T with output (S + diag(u) k v^T)^T r per head, the
     per-head RMS scale, weight g and silu(gate), over the step's rows of each sequence in turn.
-    r, k, v, d, gate: float32 [T, heads * dim] (w = exp(-exp(d + w0))); state float32
+    r, k, v, d, gate: float32 [T, heads * dim] (w = exp(-exp(d + w0))), or partial sums [parts, T, heads * dim] of
+    products split along k (r, k, v, gate with one split, d with its own); state float32
     [slots, heads * dim * dim + W]: each head's S as [value channel][key channel], then the
     last mixer input row, which this kernel replaces by h_in's last row of each sequence."""
     HD = n_heads * dim
     _dev(r, k, v, d, gate, w0, u, g, state, h_in, ctx.slots, ctx.cu_dev)
     for t, name in ((r, "r"), (k, "k"), (v, "v"), (d, "d"), (gate, "gate")):
-        _need(t.dtype == torch.float32 and t.dim() == 2 and t.shape == (ctx.n_tokens, HD), f"wkv_scan: {name} must be float32 [T, heads * dim]")
+        _need(t.dtype == torch.float32 and t.dim() in (2, 3) and tuple(t.shape[-2:]) == (ctx.n_tokens, HD),
+              f"wkv_scan: {name} must be float32 [T, heads * dim] or parts of it")
+    parts, part_stride = _parts(r)
+    for t in (k, v, gate):
+        _need(_parts(t) == (parts, part_stride), "wkv_scan: r, k, v and gate must be split alike")
+    d_parts, d_part_stride = _parts(d)
     for t, name in ((w0, "w0"), (u, "u"), (g, "g")):
         _need(t.dtype == torch.float32 and t.numel() == HD, f"wkv_scan: {name} must be float32 [heads * dim]")
     W = h_in.shape[1]
     _need(h_in.dtype == torch.float32 and h_in.shape == (ctx.n_tokens, W), "wkv_scan: h_in must be float32 [T, W]")
     _need(state.dtype == torch.float32 and state.dim() == 2 and state.shape[1] == HD * dim + W, "wkv_scan: state must be float32 [slots, heads * dim * dim + W]")
     _need(ctx.cu_dev is not None or ctx.n_tokens == ctx.batch, "wkv_scan: a step of several tokens a sequence needs the token offsets")
-    _need(6 * 16 * dim * 4 <= 65536, f"wkv_scan: head size {dim} is too large")
+    _need(6 * dim * 4 <= 65536, f"wkv_scan: head size {dim} is too large")
     y = torch.empty((ctx.n_tokens, HD), dtype=out_dtype, device=r.device)
-    _check(_lib().llogos_wkv_scan(_p(y), _DT[out_dtype], _p(r), _p(k), _p(v), _p(d), _p(gate), HD, _p(w0), _p(u), _p(g),
+    col_blocks = scan_column_blocks(ctx.n_tokens, ctx.batch, n_heads, dim) if not ctx.is_decode else 1
+    o_raw = torch.empty((ctx.n_tokens, HD), dtype=torch.float32, device=r.device) if col_blocks > 1 else None
+    _check(_lib().llogos_wkv_scan(_p(y), _DT[out_dtype], _p(r), _p(k), _p(v), _p(d), _p(gate), HD, parts, ctypes.c_longlong(part_stride),
+                                  d_parts, ctypes.c_longlong(d_part_stride), _p(w0), _p(u), _p(g),
                                   ctypes.c_float(eps), _p(state), ctypes.c_longlong(state.stride(0)), ctypes.c_longlong(HD * dim),
-                                  _p(h_in), W, _p(ctx.slots), _p(ctx.cu_dev), ctx.batch, n_heads, dim, _stream()), "wkv_scan")
+                                  _p(h_in), W, _p(ctx.slots), _p(ctx.cu_dev), ctx.batch, n_heads, dim, ctx.n_tokens, col_blocks,
+                                  _p(o_raw), _stream()), "wkv_scan")
     return y
+
+
+SCAN_COLUMN_BLOCKS = 0       # 0: chosen by the step; 1, 2, 4, ... force the number of blocks a head (tests)
+
+
+def scan_column_blocks(n_tokens: int, batch: int, n_heads: int, dim: int, n_cus: Optional[int] = None) -> int:
+    """Blocks that share a head's state columns in the recurrence over a prompt.  A block's waves sit on one
+    compute unit, which issues every token's instructions for all of them in turn: with (sequence, head)
+    pairs fewer than compute units, a head's columns go to several blocks (a power of two, at least 16
+    columns each, as many as fill the units) and the head norm to a kernel of its own.  Not for short
+    steps, where the second kernel costs more than it saves."""
+    if SCAN_COLUMN_BLOCKS:
+        return SCAN_COLUMN_BLOCKS
+    n_cus = n_cus or compute_units()
+    blocks, pairs = 1, batch * n_heads
+    if n_tokens < 64 * batch:
+        return 1
+    while blocks * 2 * pairs <= n_cus and dim // (blocks * 2) >= 16 and dim % (blocks * 2) == 0:
+        blocks *= 2
+    return blocks
 
 
 def sandwich_norm(x: torch.Tensor, a: torch.Tensor, post_w: torch.Tensor, next_w: Optional[torch.Tensor], eps: float,

@@ -71,11 +71,12 @@ class WKV(Mixer):
         prev = state[:, self.inner * self.head_dim:]
         m = K.token_shift(ctx, h, self.mu, prev, self.rt.dtype)                # [5, T, hidden]
         mark(ctx, "shift")
-        # (a product may come as float32 partial sums of a split along k: the activation adds them itself)
-        plain = lambda p: K.sum_parts(p, None, f32)
-        r, k, v, g = (plain(lin.product(m[i], f32_ok=True)) for i, lin in enumerate((self.r, self.k, self.v, self.g)))
+        # (a product may come as float32 partial sums of a split along k: the activation and the recurrence add them
+        # themselves; r, k, v, g have one shape and so one split)
+        as_f32 = lambda p: (p[0] if p.dim() == 3 and p.shape[0] == 1 else p) if p.dtype == f32 else K.sum_parts(p, None, f32)
+        r, k, v, g = (as_f32(lin.product(m[i], f32_ok=True)) for i, lin in enumerate((self.r, self.k, self.v, self.g)))
         low = K.activation(self.w1.product(m[4], f32_ok=True), "tanh", self.rt.dtype)
-        d = plain(self.w2.product(low, f32_ok=True))
+        d = as_f32(self.w2.product(low, f32_ok=True))
         mark(ctx, "projections")
         y = K.wkv_scan(ctx, r, k, v, d, g, self.w0, self.u, self.norm_w, self.eps, state, self.n_heads, self.head_dim,
                        h, self.rt.dtype)
