@@ -161,7 +161,12 @@ __device__ __forceinline__ float dpp_add(float x, int ctrl_index) {
 
 // PP: parts of a column (a power of two up to 16); EXACT: every thread has exactly RPT rows (D = PP * RPT), read
 // as float4s without a bound check.  Both are template arguments so that a token's loop has no branch.
-template <int RPT, int PP, bool EXACT, typename TO>
+// MODE 0: a sequence's part of the step from the cached state to the cached state.  Long prompts of few
+// sequences are cut into segments that run side by side: MODE 1 takes a segment from a zero state and leaves its
+// end state and the product of its decays (no outputs); wkv_combine_kernel chains those into every segment's true
+// initial state and the sequence's final state, S_init[s + 1] = diag(prod decay_s) S_init[s] + S_local[s]; MODE 2
+// runs the segment again from its initial state for the outputs, token by token as MODE 0 would.
+template <int RPT, int PP, bool EXACT, int MODE, typename TO>
 __global__ void wkv_scan_kernel(TO* __restrict__ y, const float* __restrict__ r, const float* __restrict__ k,
                                 const float* __restrict__ v, const float* __restrict__ d, const float* __restrict__ gate,
                                 int ld, int parts, size_t part_stride, int d_parts, size_t d_part_stride,
@@ -170,17 +175,36 @@ __global__ void wkv_scan_kernel(TO* __restrict__ y, const float* __restrict__ r,
                                 float* __restrict__ state, size_t state_stride, size_t prev_offset,
                                 const float* __restrict__ h_in, int W,
                                 const int* __restrict__ slots, const int* __restrict__ cu,
-                                int H, int D, int rpt, int chunk, int Dc, float* __restrict__ o_raw) {
+                                int H, int D, int rpt, int chunk, int Dc, float* __restrict__ o_raw,
+                                int col_blocks, int n_seg, int seg_len, float* __restrict__ seg_state,
+                                float* __restrict__ seg_decay) {
     constexpr int P = PP;
     extern __shared__ float smem[];
     const int seq = blockIdx.x, head = blockIdx.y;
-    const int first = cu ? cu[seq] : seq, count = cu ? cu[seq + 1] - first : 1;
+    const int cbi = blockIdx.z % col_blocks, seg = blockIdx.z / col_blocks;
+    const int first0 = cu ? cu[seq] : seq, count0 = cu ? cu[seq + 1] - first0 : 1;
+    const int first = first0 + (MODE ? seg * seg_len : 0);
+    const int count = MODE ? min(seg_len, count0 - seg * seg_len) : count0;
     const int tid = threadIdx.x, nthreads = blockDim.x;
     // the block's columns of S: all D, or, with several blocks a head (long prompts of few sequences: a
-    // compute unit issues a token's instructions for all of a block's waves), Dc of them from blockIdx.z * Dc on
-    const int j = blockIdx.z * Dc + tid / P, part = tid % P;
+    // compute unit issues a token's instructions for all of a block's waves), Dc of them from cbi * Dc on
+    const int j = cbi * Dc + tid / P, part = tid % P;
     const bool active = tid / P < Dc && j < D;
     const int i0 = part * rpt;
+    float* seg_S = MODE ? seg_state + ((((size_t)seq * n_seg + seg) * H + head) * D + (active ? j : 0)) * D + i0 : nullptr;
+    float* seg_P = MODE ? seg_decay + (((size_t)seq * n_seg + seg) * H + head) * D + i0 : nullptr;
+    const bool keeps_decay = MODE == 1 && cbi == 0 && tid / P == 0;      // one column's threads keep the decays' product
+    if (MODE && count <= 0) {
+        if (MODE == 1) {                                   // a segment beyond the sequence's end: nothing added, nothing decayed
+#pragma unroll
+            for (int m = 0; m < RPT; ++m)
+                if (m < rpt && i0 + m < D) {
+                    if (active) seg_S[m] = 0.f;
+                    if (keeps_decay) seg_P[m] = 1.f;
+                }
+        }
+        return;
+    }
     float* s_r = smem;                          // [chunk][D]
     float* s_k = s_r + chunk * D;
     float* s_w = s_k + chunk * D;
@@ -191,12 +215,13 @@ __global__ void wkv_scan_kernel(TO* __restrict__ y, const float* __restrict__ r,
     float* S = row + ((size_t)head * D + (active ? j : 0)) * D + i0;
     const size_t col0 = (size_t)head * D;
 
-    float s[RPT], ur[RPT];
+    float s[RPT], ur[RPT], pw[RPT];
 #pragma unroll
     for (int m = 0; m < RPT; ++m) {
         const bool ok = active && m < rpt && i0 + m < D;
-        s[m] = ok ? S[m] : 0.f;
+        s[m] = !ok || MODE == 1 ? 0.f : (MODE == 2 ? seg_S[m] : S[m]);
         ur[m] = ok ? u[col0 + i0 + m] : 0.f;
+        pw[m] = 1.f;
     }
 
     // a chunk's values on their way: element e = tid + a * nthreads of the chunk's [n][D]
@@ -239,6 +264,16 @@ __global__ void wkv_scan_kernel(TO* __restrict__ y, const float* __restrict__ r,
             const float* kk = smem + o_k + at;
             const float* ww = smem + o_w + at;
             const float vj = active ? smem[3 * chunk * D + c * D + j] : 0.f;
+            if (MODE == 1) {                               // the state alone
+#pragma unroll
+                for (int m = 0; m < RPT; ++m) {
+                    if (EXACT || (m < rpt && i0 + m < D)) {
+                        s[m] = fmaf(ww[m], s[m], kk[m] * vj);
+                        pw[m] *= ww[m];
+                    }
+                }
+                continue;
+            }
             float acc = 0.f;
             if (EXACT) {
 #pragma unroll
@@ -272,11 +307,12 @@ __global__ void wkv_scan_kernel(TO* __restrict__ y, const float* __restrict__ r,
             if (P >= 16) acc = dpp_add(acc, 3);
             if (active && part == 0) smem[5 * chunk * D + c * D + j] = acc;
         }
+        if (MODE == 1) continue;
         __syncthreads();
         if (o_raw) {
             // several blocks a head: the raw outputs of this block's columns; head_norm_gate_kernel norms the head
             for (int e = tid; e < n * Dc; e += nthreads) {
-                const int c = e / Dc, jj = blockIdx.z * Dc + e % Dc;
+                const int c = e / Dc, jj = cbi * Dc + e % Dc;
                 if (jj < D) o_raw[(size_t)(first + c0 + c) * H * D + col0 + jj] = s_o[c * D + jj];
             }
             continue;
@@ -298,10 +334,33 @@ __global__ void wkv_scan_kernel(TO* __restrict__ y, const float* __restrict__ r,
     }
 #pragma unroll
     for (int m = 0; m < RPT; ++m)
-        if (active && m < rpt && i0 + m < D) S[m] = s[m];
-    if (head == 0 && blockIdx.z == 0 && h_in) {
-        const float* last = h_in + (size_t)(first + count - 1) * W;
+        if (m < rpt && i0 + m < D) {
+            if (active && MODE == 0) S[m] = s[m];
+            if (active && MODE == 1) seg_S[m] = s[m];
+            if (keeps_decay) seg_P[m] = pw[m];
+        }
+    if (MODE != 1 && head == 0 && blockIdx.z == 0 && h_in) {
+        const float* last = h_in + (size_t)(first0 + count0 - 1) * W;
         for (int c = tid; c < W; c += nthreads) row[prev_offset + c] = last[c];
+    }
+}
+
+// The segments' local end states chained: seg_state[seg] <- the state the segment starts from, and the cached state
+// <- the state after the last segment.  One block a (sequence, head); a thread owns elements (j, i) of S.
+__global__ void wkv_combine_kernel(float* __restrict__ state, size_t state_stride, const int* __restrict__ slots,
+                                   float* __restrict__ seg_state, const float* __restrict__ seg_decay, int H, int D, int n_seg) {
+    const int seq = blockIdx.x, head = blockIdx.y;
+    float* S = state + (size_t)slots[seq] * state_stride + (size_t)head * D * D;
+    for (int e = threadIdx.x; e < D * D; e += blockDim.x) {
+        const int i = e % D;
+        float cur = S[e];
+        for (int sg = 0; sg < n_seg; ++sg) {
+            const size_t at = ((size_t)seq * n_seg + sg) * H + head;
+            const float local = seg_state[at * D * D + e];
+            seg_state[at * D * D + e] = cur;
+            cur = fmaf(seg_decay[at * D + i], cur, local);
+        }
+        S[e] = cur;
     }
 }
 
@@ -331,12 +390,17 @@ LLOGOS_EXPORT int llogos_wkv_scan(void* y, int out_dtype, const float* r, const 
                                   long long d_part_stride, const float* w0, const float* u, const float* g, float eps,
                                   float* state, long long state_stride, long long prev_offset, const float* h_in, int W,
                                   const int* slots, const int* cu, int B, int H, int D, int T, int col_blocks, float* o_raw,
+                                  int n_seg, int seg_len, float* seg_state, float* seg_decay, int rows_hint,
                                   hipStream_t stream) {
+    if (n_seg < 1 || (n_seg > 1 && (!cu || seg_len < 1 || !seg_state || !seg_decay))) return LLOGOS_BAD_ARGUMENT;
     if (B <= 0 || H <= 0 || D <= 0 || ld < H * D || parts < 1 || d_parts < 1 || col_blocks < 1 || (col_blocks > 1 && !o_raw)) return LLOGOS_BAD_ARGUMENT;
     // rows a thread: the fewest of 4, 16, 64 with which a column's parts (a power of two, at most 16: one
     // row of lanes) make a block of at most 1024 threads
+    // (rows_hint 16: the caller has enough blocks to fill the machine and wants the threads with more rows each,
+    // which spend fewer of their instructions on fetching r, k and the decay and on adding up)
     int rpt_max = 0, P = 1;
     for (int cand : {4, 16, 64}) {
+        if (cand < rows_hint) continue;
         P = 1;
         while (P * cand < D) P <<= 1;
         if (P <= 16 && (long long)((D * P + kWave - 1) / kWave * kWave) <= 1024) { rpt_max = cand; break; }
@@ -353,22 +417,31 @@ LLOGOS_EXPORT int llogos_wkv_scan(void* y, int out_dtype, const float* r, const 
     const size_t smem = (size_t)6 * chunk * D * sizeof(float);
     if (smem > 65536) return LLOGOS_UNSUPPORTED;
     if (col_blocks == 1) o_raw = nullptr;
-    dim3 grid(B, H, col_blocks);
+    dim3 grid(B, H, col_blocks * n_seg);
 #define ARGS(TO) ((TO*)y, r, k, v, d, gate, ld, parts, (size_t)part_stride, d_parts, (size_t)d_part_stride, w0, u, g, eps, \
-        state, (size_t)state_stride, (size_t)prev_offset, h_in, W, slots, cu, H, D, rpt, chunk, Dc, o_raw)
+        state, (size_t)state_stride, (size_t)prev_offset, h_in, W, slots, cu, H, D, rpt, chunk, Dc, o_raw, col_blocks, n_seg, \
+        seg_len, seg_state, seg_decay)
     const bool exact = rpt == rpt_max && P * rpt == D;
-#define SCAN(RPT, PP, TO) do { if (exact) wkv_scan_kernel<RPT, PP, true, TO><<<grid, threads, smem, stream>>> ARGS(TO); \
-                               else wkv_scan_kernel<RPT, PP, false, TO><<<grid, threads, smem, stream>>> ARGS(TO); } while (0)
+#define SCAN1(RPT, PP, EX, TO) do { \
+        if (n_seg == 1) wkv_scan_kernel<RPT, PP, EX, 0, TO><<<grid, threads, smem, stream>>> ARGS(TO); \
+        else { \
+            wkv_scan_kernel<RPT, PP, EX, 1, float><<<grid, threads, smem, stream>>> ARGS(float); \
+            wkv_combine_kernel<<<dim3(B, H), 256, 0, stream>>>(state, (size_t)state_stride, slots, seg_state, seg_decay, H, D, n_seg); \
+            wkv_scan_kernel<RPT, PP, EX, 2, TO><<<grid, threads, smem, stream>>> ARGS(TO); \
+        } } while (0)
+#define SCAN(RPT, PP, TO) do { if (exact) SCAN1(RPT, PP, true, TO); else SCAN1(RPT, PP, false, TO); } while (0)
 #define SCANS(TO) do { \
         if (rpt_max == 4) { if (P == 1) SCAN(4, 1, TO); else if (P == 2) SCAN(4, 2, TO); else if (P == 4) SCAN(4, 4, TO); \
                             else if (P == 8) SCAN(4, 8, TO); else SCAN(4, 16, TO); } \
-        else if (rpt_max == 16) { if (P == 8) SCAN(16, 8, TO); else SCAN(16, 16, TO); } \
+        else if (rpt_max == 16) { if (P == 1) SCAN(16, 1, TO); else if (P == 2) SCAN(16, 2, TO); else if (P == 4) SCAN(16, 4, TO); \
+                                  else if (P == 8) SCAN(16, 8, TO); else SCAN(16, 16, TO); } \
         else { if (P == 4) SCAN(64, 4, TO); else return LLOGOS_UNSUPPORTED; } } while (0)
     if (out_dtype == DT_F32) SCANS(float);
     else if (out_dtype == DT_BF16) SCANS(bf16_t);
     else return LLOGOS_BAD_ARGUMENT;
 #undef SCANS
 #undef SCAN
+#undef SCAN1
 #undef ARGS
     if (o_raw) {
         const int n = T * H, waves = 4;

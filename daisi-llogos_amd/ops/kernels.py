@@ -378,34 +378,56 @@ def wkv_scan(ctx, r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, d: torch.Te
     _need(ctx.cu_dev is not None or ctx.n_tokens == ctx.batch, "wkv_scan: a step of several tokens a sequence needs the token offsets")
     _need(6 * dim * 4 <= 65536, f"wkv_scan: head size {dim} is too large")
     y = torch.empty((ctx.n_tokens, HD), dtype=out_dtype, device=r.device)
-    col_blocks = scan_column_blocks(ctx.n_tokens, ctx.batch, n_heads, dim) if not ctx.is_decode else 1
+    rows, col_blocks, n_seg = scan_plan(ctx.batch, n_heads, dim, None if ctx.is_decode else
+                                        max(ctx.cu_seqlens[i + 1] - ctx.cu_seqlens[i] for i in range(ctx.batch)))
     o_raw = torch.empty((ctx.n_tokens, HD), dtype=torch.float32, device=r.device) if col_blocks > 1 else None
+    seg_len, seg_state, seg_decay = 0, None, None
+    if n_seg > 1:
+        longest = max(ctx.cu_seqlens[i + 1] - ctx.cu_seqlens[i] for i in range(ctx.batch))
+        seg_len = -(-(-(-longest // n_seg)) // 16) * 16                  # whole chunks of the kernel
+        seg_state = torch.empty((ctx.batch, n_seg, n_heads, dim, dim), dtype=torch.float32, device=r.device)
+        seg_decay = torch.empty((ctx.batch, n_seg, n_heads, dim), dtype=torch.float32, device=r.device)
     _check(_lib().llogos_wkv_scan(_p(y), _DT[out_dtype], _p(r), _p(k), _p(v), _p(d), _p(gate), HD, parts, ctypes.c_longlong(part_stride),
                                   d_parts, ctypes.c_longlong(d_part_stride), _p(w0), _p(u), _p(g),
                                   ctypes.c_float(eps), _p(state), ctypes.c_longlong(state.stride(0)), ctypes.c_longlong(HD * dim),
                                   _p(h_in), W, _p(ctx.slots), _p(ctx.cu_dev), ctx.batch, n_heads, dim, ctx.n_tokens, col_blocks,
-                                  _p(o_raw), _stream()), "wkv_scan")
+                                  _p(o_raw), n_seg, seg_len, _p(seg_state), _p(seg_decay), rows, _stream()), "wkv_scan")
     return y
 
 
 SCAN_COLUMN_BLOCKS = 0       # 0: chosen by the step; 1, 2, 4, ... force the number of blocks a head (tests)
+SCAN_SEGMENTS = 0            # 0: chosen by the step; 1, 2, 3, ... force the number of segments of a prompt (tests)
 
 
-def scan_column_blocks(n_tokens: int, batch: int, n_heads: int, dim: int, n_cus: Optional[int] = None) -> int:
-    """Blocks that share a head's state columns in the recurrence over a prompt.  A block's waves sit on one
-    compute unit, which issues every token's instructions for all of them in turn: with (sequence, head)
-    pairs fewer than compute units, a head's columns go to several blocks (a power of two, at least 16
-    columns each, as many as fill the units) and the head norm to a kernel of its own.  Not for short
-    steps, where the second kernel costs more than it saves."""
-    if SCAN_COLUMN_BLOCKS:
-        return SCAN_COLUMN_BLOCKS
+def scan_plan(batch: int, n_heads: int, dim: int, longest: Optional[int], n_cus: Optional[int] = None) -> Tuple[int, int, int]:
+    """(rows of the state a thread, blocks a head, segments a prompt) for the recurrence; `longest` is the most
+    tokens a sequence brings (None: a single-token step).  Measured on the MI355X (64 heads of 64, one prompt of
+    2,048 tokens): a block a head with 4 rows a thread 1,014 us, its columns over 4 blocks 550 us (a chain of
+    2,048 dependent steps of 270 ns, whatever else is done); cut into 4 to 16 segments that run side by side
+    (each twice: once for its end state from zero, once for its outputs from its true initial state) 455 us, no
+    longer bound by the chain but by the instructions a token costs a thread, of which with 4 rows a thread two
+    thirds fetch r, k and the decay and add up the parts; hence 16 rows a thread wherever the blocks fill the
+    machine without the finer split.
+    Segments: as many as bring the waves to about six a SIMD, of at least 128 tokens, at most 16."""
     n_cus = n_cus or compute_units()
-    blocks, pairs = 1, batch * n_heads
-    if n_tokens < 64 * batch:
-        return 1
-    while blocks * 2 * pairs <= n_cus and dim // (blocks * 2) >= 16 and dim % (blocks * 2) == 0:
-        blocks *= 2
-    return blocks
+    simds = 4 * n_cus
+    wide = dim % 16 == 0 and dim <= 256                              # 16 rows a thread tile the head exactly
+    waves16 = batch * n_heads * max(1, (dim * max(1, dim // 16) + 63) // 64) if wide else 0
+    n_seg = 1
+    if longest is not None:
+        base = waves16 if wide else batch * n_heads * max(1, (dim * 16 + 63) // 64)
+        n_seg = max(1, min(16, longest // 128, -(-(6 * simds) // max(1, base))))
+    if SCAN_SEGMENTS and longest is not None:
+        n_seg = SCAN_SEGMENTS
+    if SCAN_COLUMN_BLOCKS and longest is not None:
+        return 4, SCAN_COLUMN_BLOCKS, n_seg
+    if wide and waves16 * n_seg >= 2 * simds:
+        return 16, 1, n_seg
+    blocks, pairs = 1, batch * n_heads * n_seg
+    if longest is not None and longest >= 64:
+        while blocks * 2 * pairs <= n_cus and dim // (blocks * 2) >= 16 and dim % (blocks * 2) == 0:
+            blocks *= 2
+    return 4, blocks, n_seg
 
 
 def sandwich_norm(x: torch.Tensor, a: torch.Tensor, post_w: torch.Tensor, next_w: Optional[torch.Tensor], eps: float,
