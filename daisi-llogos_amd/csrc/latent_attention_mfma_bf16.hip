@@ -113,15 +113,17 @@ __global__ __launch_bounds__(kLatentWaves* kWave) void latent_attn_kernel(
         const int key0 = pg * kPageTokens;
         lf32x4 s[4];
 #pragma unroll
-        for (int rb = 0; rb < 4; ++rb) {
-            s[rb] = lf32x4{0.f, 0.f, 0.f, 0.f};
+        for (int rb = 0; rb < 4; ++rb) s[rb] = lf32x4{0.f, 0.f, 0.f, 0.f};
+        // (the four blocks of keys side by side: four loads in flight and four independent chains of products)
 #pragma unroll
-            for (int sk = 0; sk < KS; ++sk) {
-                if (sk < ksteps) {
-                    // block rb of the page, dimensions 32 sk + 8 g ..: beyond the row's end nothing is there
-                    const lbf16x8 kf = (4 * sk + g < octs) ? frag_load(kpage + (size_t)(rb * octs + 4 * sk) * 128) : frag_zero();
-                    s[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[sk], s[rb], 0, 0, 0);
-                }
+        for (int sk = 0; sk < KS; ++sk) {
+            if (sk < ksteps) {
+                lbf16x8 kf[4];
+#pragma unroll
+                for (int rb = 0; rb < 4; ++rb)      // block rb of the page, dimensions 32 sk + 8 g ..: beyond the row's end nothing is there
+                    kf[rb] = (4 * sk + g < octs) ? frag_load(kpage + (size_t)(rb * octs + 4 * sk) * 128) : frag_zero();
+#pragma unroll
+                for (int rb = 0; rb < 4; ++rb) s[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[rb], qf[sk], s[rb], 0, 0, 0);
             }
         }
         // softmax of the page: this lane holds, for its column, keys key0 + 16 g + 4 rb + r
@@ -161,20 +163,32 @@ __global__ __launch_bounds__(kLatentWaves* kWave) void latent_attn_kernel(
         }
         // values of keys that are not written yet are zeroed (whatever the page held before times 0 must be 0)
         const int valid = pos_hi + 1 - key0;
+        // (four tiles of value dimensions at a time: eight loads in flight before the first product)
 #pragma unroll
-        for (int db = 0; db < DVT; ++db) {
-            if (db < dvt) {
-                lf32x4 a = acc[db];
+        for (int d0 = 0; d0 < DVT; d0 += 4) {
+            if (d0 < dvt) {
+                lbf16x8 v0[4], v1[4];
 #pragma unroll
-                for (int r = 0; r < 4; ++r) a[r] *= corr;
-                lbf16x8 v0 = frag_load(vpage + 512 * (2 * db)), v1 = frag_load(vpage + 512 * (2 * db + 1));
-                if (valid < kPageTokens) {
-                    v0 = first_n(v0, valid - 16 * g);
-                    v1 = first_n(v1, valid - 16 * g - 8);
+                for (int e = 0; e < 4; ++e) {
+                    const bool on = d0 + e < DVT && d0 + e < dvt;
+                    v0[e] = on ? frag_load(vpage + 512 * (2 * (d0 + e))) : frag_zero();
+                    v1[e] = on ? frag_load(vpage + 512 * (2 * (d0 + e) + 1)) : frag_zero();
+                    if (valid < kPageTokens) {
+                        v0[e] = first_n(v0[e], valid - 16 * g);
+                        v1[e] = first_n(v1[e], valid - 16 * g - 8);
+                    }
                 }
-                a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v0, pf[0], a, 0, 0, 0);
-                a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v1, pf[1], a, 0, 0, 0);
-                acc[db] = a;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    if (d0 + e < DVT) {
+                        lf32x4 a = acc[d0 + e];
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) a[r] *= corr;
+                        a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v0[e], pf[0], a, 0, 0, 0);
+                        a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v1[e], pf[1], a, 0, 0, 0);
+                        acc[d0 + e] = a;
+                    }
+                }
             }
         }
     }
