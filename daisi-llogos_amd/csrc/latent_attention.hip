@@ -135,6 +135,79 @@ __global__ __launch_bounds__(256) void head_products_kernel(TO* __restrict__ out
     }
 }
 
+// The same for steps of up to 16 rows, where the tiles above would be nearly empty: the rows of a head go to
+// LDS once, a thread owns an output n and a quarter of k and streams its part of the head's matrix, which for
+// this kernel is stored k-major, w_kn [H, K, N], so that neighbouring threads read neighbouring values; the four
+// quarters are added in a fixed order.  TMAX: the rows
+// rounded up to 1, 2, 4, 8 or 16 (rows that are not there are zeros in LDS).
+template <int TMAX, typename TA, typename TW, typename TO>
+__global__ __launch_bounds__(256) void head_products_few_kernel(TO* __restrict__ out, int ldo, int o_head, const TA* __restrict__ a, int lda, int a_head,
+                                         const TW* __restrict__ w_kn, int M, int N, int K) {
+    // LDS: the head's rows as [k][TMAX] (one or two 16-byte reads bring every row's value of a k), then the four
+    // k-groups' sums [4][64][TMAX]
+    extern __shared__ float rows_lds[];
+    float* sums = rows_lds + (size_t)K * TMAX;
+    const int h = blockIdx.y, nl = threadIdx.x & 63, kg = threadIdx.x >> 6, n = blockIdx.x * 64 + nl;
+#pragma unroll 4
+    for (int e = threadIdx.x; e < TMAX * K; e += blockDim.x) {      // (neighbouring threads read neighbouring k of a row)
+        const int t = e / K, k = e % K;
+        rows_lds[k * TMAX + t] = t < M ? load_f32(a + (size_t)t * lda + (size_t)h * a_head + k) : 0.f;
+    }
+    __syncthreads();
+    float acc[TMAX];
+#pragma unroll
+    for (int t = 0; t < TMAX; ++t) acc[t] = 0.f;
+    // this thread: output n, the k of its group: kg, kg + 4, ... (the groups' loads of w lie 4 rows apart)
+    if (n < N) {
+        const TW* wp = w_kn + (size_t)h * K * N + n;
+        for (int k0 = kg; k0 < K; k0 += 16) {
+            float wv[4];
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) wv[kk] = k0 + 4 * kk < K ? load_f32(wp + (size_t)(k0 + 4 * kk) * N) : 0.f;
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) {
+                const int k = min(k0 + 4 * kk, K - 1);                   // (beyond the end: wv is 0)
+#pragma unroll
+                for (int t = 0; t < TMAX; ++t) acc[t] = fmaf(rows_lds[k * TMAX + t], wv[kk], acc[t]);
+            }
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < TMAX; ++t) sums[(kg * 64 + nl) * TMAX + t] = acc[t];
+    __syncthreads();
+    if (kg == 0 && n < N) {
+#pragma unroll
+        for (int t = 0; t < TMAX; ++t) {
+            const float v = ((sums[(0 * 64 + nl) * TMAX + t] + sums[(1 * 64 + nl) * TMAX + t]) + sums[(2 * 64 + nl) * TMAX + t]) + sums[(3 * 64 + nl) * TMAX + t];
+            if (t < M) store_f32(out + (size_t)t * ldo + (size_t)h * o_head + n, v);
+        }
+    }
+}
+
+LLOGOS_EXPORT int llogos_head_products_few(void* out, int out_dtype, int ldo, int o_head, const void* a, int a_dtype, int lda,
+                                           int a_head, const void* w_kn, int w_dtype, int M, int H, int N, int K,
+                                           hipStream_t stream) {
+    if (M <= 0 || M > 16 || H <= 0 || N <= 0 || K <= 0) return LLOGOS_BAD_ARGUMENT;
+    int tmax = 1;
+    while (tmax < M) tmax <<= 1;
+    const size_t smem = (size_t)tmax * (K + 256) * sizeof(float);
+    if (smem > 65536) return LLOGOS_UNSUPPORTED;
+    const int threads = 256;
+    dim3 grid((N + 63) / 64, H);
+#define HPF(TM, TA, TW, TO) head_products_few_kernel<TM, TA, TW, TO><<<grid, threads, smem, stream>>>((TO*)out, ldo, o_head, \
+        (const TA*)a, lda, a_head, (const TW*)w_kn, M, N, K)
+#define HPT(TA, TW, TO) do { if (tmax == 1) HPF(1, TA, TW, TO); else if (tmax == 2) HPF(2, TA, TW, TO); else if (tmax == 4) HPF(4, TA, TW, TO); \
+                             else if (tmax == 8) HPF(8, TA, TW, TO); else HPF(16, TA, TW, TO); } while (0)
+    if (a_dtype == DT_F32 && w_dtype == DT_F32 && out_dtype == DT_F32) HPT(float, float, float);
+    else if (a_dtype == DT_F32 && w_dtype == DT_BF16 && out_dtype == DT_BF16) HPT(float, bf16_t, bf16_t);
+    else if (a_dtype == DT_BF16 && w_dtype == DT_BF16 && out_dtype == DT_BF16) HPT(bf16_t, bf16_t, bf16_t);
+    else if (a_dtype == DT_BF16 && w_dtype == DT_BF16 && out_dtype == DT_F32) HPT(bf16_t, bf16_t, float);
+    else return LLOGOS_BAD_ARGUMENT;
+#undef HPT
+#undef HPF
+    return LLOGOS_LAUNCH_CHECK();
+}
+
 LLOGOS_EXPORT int llogos_head_products(void* out, int out_dtype, int ldo, int o_head, const void* a, int a_dtype, int lda,
                                        int a_head, const void* w, int w_dtype, int M, int H, int N, int K, hipStream_t stream) {
     if (M <= 0 || H <= 0 || N <= 0 || K <= 0) return LLOGOS_BAD_ARGUMENT;

@@ -221,23 +221,33 @@ __global__ __launch_bounds__(kLatentWaves* kWave) void latent_attn_kernel(
 
 // out[col, d] = sum_s acc_s[d] 2^(m_s - M) / sum_s l_s 2^(m_s - M), M the largest m_s (splits that saw
 // no key have m = -inf and l = 0 and count for nothing).
+constexpr int kMergeSplits = 16;      // splits whose partial results a thread asks for at once (the wrapper makes no more)
+
 __global__ void latent_merge_kernel(bf16_t* __restrict__ out, int dv, int dvp, const float* __restrict__ ws_ml,
                                     const float* __restrict__ ws_acc, int splits, int total_cols) {
     const int col = blockIdx.x;
-    float M = -INFINITY;
-    for (int s = 0; s < splits; ++s) M = fmaxf(M, ws_ml[((size_t)s * total_cols + col) * 2]);
-    float L = 0.f;
-    for (int s = 0; s < splits; ++s) {
-        const float ms = ws_ml[((size_t)s * total_cols + col) * 2];
-        if (ms != -INFINITY) L += ws_ml[((size_t)s * total_cols + col) * 2 + 1] * __builtin_amdgcn_exp2f(ms - M);
+    float ms[kMergeSplits], ls[kMergeSplits];
+#pragma unroll
+    for (int s = 0; s < kMergeSplits; ++s) {
+        ms[s] = s < splits ? ws_ml[((size_t)s * total_cols + col) * 2] : -INFINITY;
+        ls[s] = s < splits ? ws_ml[((size_t)s * total_cols + col) * 2 + 1] : 0.f;
+    }
+    float M = -INFINITY, L = 0.f;
+#pragma unroll
+    for (int s = 0; s < kMergeSplits; ++s) M = fmaxf(M, ms[s]);
+#pragma unroll
+    for (int s = 0; s < kMergeSplits; ++s) {
+        ms[s] = ms[s] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms[s] - M);       // the split's weight
+        L = fmaf(ls[s], ms[s], L);
     }
     const float inv = L > 0.f ? 1.0f / L : 0.f;
     for (int d = threadIdx.x; d < dv; d += blockDim.x) {
+        float part[kMergeSplits];
+#pragma unroll
+        for (int s = 0; s < kMergeSplits; ++s) part[s] = s < splits ? ws_acc[((size_t)s * total_cols + col) * dvp + d] : 0.f;
         float a = 0.f;
-        for (int s = 0; s < splits; ++s) {
-            const float ms = ws_ml[((size_t)s * total_cols + col) * 2];
-            if (ms != -INFINITY) a = fmaf(ws_acc[((size_t)s * total_cols + col) * dvp + d], __builtin_amdgcn_exp2f(ms - M), a);
-        }
+#pragma unroll
+        for (int s = 0; s < kMergeSplits; ++s) a = fmaf(part[s], ms[s], a);
         out[(size_t)col * dv + d] = f32_to_bf16(a * inv);
     }
 }
@@ -257,7 +267,7 @@ LLOGOS_EXPORT int llogos_latent_attn_bf16(void* out, int dv, const void* q, cons
                                           int n_tiles, int splits, int pages_per_split, float* workspace,
                                           long long workspace_floats, hipStream_t stream) {
     if (T <= 0 || batch <= 0 || n_heads <= 0 || row <= 0 || row % 16 || dv <= 0 || dv > row || n_tiles <= 0) return LLOGOS_BAD_ARGUMENT;
-    if (splits < 1 || pages_per_split < 1 || (!cu && T != batch)) return LLOGOS_BAD_ARGUMENT;
+    if (splits < 1 || splits > kMergeSplits || pages_per_split < 1 || (!cu && T != batch)) return LLOGOS_BAD_ARGUMENT;
     if (row > 576) return LLOGOS_UNSUPPORTED;
     const int total_cols = T * n_heads, dvp = (dv + 15) / 16 * 16;
     float *ws_ml = nullptr, *ws_acc = nullptr;
@@ -274,6 +284,6 @@ LLOGOS_EXPORT int llogos_latent_attn_bf16(void* out, int dv, const void* q, cons
     else if (row <= 256) LAT(8, 16);
     else LAT(18, 36);
 #undef LAT
-    if (splits > 1) latent_merge_kernel<<<total_cols, 128, 0, stream>>>((bf16_t*)out, dv, dvp, ws_ml, ws_acc, splits, total_cols);
+    if (splits > 1) latent_merge_kernel<<<total_cols, 256, 0, stream>>>((bf16_t*)out, dv, dvp, ws_ml, ws_acc, splits, total_cols);
     return LLOGOS_LAUNCH_CHECK();
 }

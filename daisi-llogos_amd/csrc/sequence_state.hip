@@ -459,48 +459,81 @@ LLOGOS_EXPORT int llogos_wkv_scan(void* y, int out_dtype, const float* r, const 
 //     v = sum of the parts of a;   x <- x + v / sqrt(mean(v^2) + eps) * wb
 //     h = x / sqrt(mean(x^2) + eps) * wn           (skipped without wn)
 // x is the float residual stream (written back), a the sublayer's output (float or bfloat16,
-// maybe in parts of a k-split product), h the rows the next sublayer reads.
-template <typename TA, typename TH>
-__global__ void sandwich_norm_kernel(float* __restrict__ x, const TA* __restrict__ a, int parts, size_t part_stride,
+// maybe in parts of a k-split product), h the rows the next sublayer reads.  A thread keeps its
+// elements of the row in registers between the two passes.
+// (A step of few rows has few blocks, and a block's time is the latency of its loads: every part of every
+// element a thread owns is asked for before the first sum, ITEMS elements a thread and up to kSandwichParts
+// parts, as rmsnorm_vec_kernel does; more parts are added by a loop behind them.)
+constexpr int kSandwichParts = 8;
+
+template <typename TA, typename TH, int ITEMS>
+__global__ __launch_bounds__(1024) void sandwich_norm_kernel(float* __restrict__ x, const TA* __restrict__ a, int parts, size_t part_stride,
                                      const float* __restrict__ wb, const float* __restrict__ wn, TH* __restrict__ h,
                                      float eps, int H) {
-    extern __shared__ float rowbuf[];
     __shared__ float red[16];
     const size_t r = blockIdx.x;
     float* xr = x + r * H;
     const TA* ar = a + r * H;
+    float v[ITEMS], xv[ITEMS], wbv[ITEMS], wnv[ITEMS], pv[ITEMS][kSandwichParts];
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it) {
+        const int i = it * blockDim.x + threadIdx.x;
+        const bool ok = i < H;
+        xv[it] = ok ? xr[i] : 0.f;
+        wbv[it] = ok ? wb[i] : 0.f;
+        wnv[it] = (ok && wn) ? wn[i] : 0.f;
+#pragma unroll
+        for (int q = 0; q < kSandwichParts; ++q) pv[it][q] = (ok && q < parts) ? load_f32(ar + q * part_stride + i) : 0.f;
+    }
     float ss = 0.f;
-    for (int i = threadIdx.x; i < H; i += blockDim.x) {
-        float v = load_f32(ar + i);
-        for (int q = 1; q < parts; ++q) v += load_f32(ar + q * part_stride + i);
-        rowbuf[i] = v;
-        ss = fmaf(v, v, ss);
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it) {
+        const int i = it * blockDim.x + threadIdx.x;
+        float t = pv[it][0];
+#pragma unroll
+        for (int q = 1; q < kSandwichParts; ++q) t += pv[it][q];            // ascending order
+        for (int q = kSandwichParts; q < parts; ++q) if (i < H) t += load_f32(ar + q * part_stride + i);
+        v[it] = t;
+        ss = fmaf(t, t, ss);
     }
     const float inv_a = 1.0f / sqrtf(block_sum(ss, red) / (float)H + eps);
     ss = 0.f;
-    for (int i = threadIdx.x; i < H; i += blockDim.x) {
-        const float v = fmaf(rowbuf[i] * inv_a, wb[i], xr[i]);
-        xr[i] = v;
-        rowbuf[i] = v;
-        ss = fmaf(v, v, ss);
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it) {
+        const int i = it * blockDim.x + threadIdx.x;
+        const float t = fmaf(v[it] * inv_a, wbv[it], xv[it]);
+        if (i < H) xr[i] = t;
+        v[it] = t;
+        ss = fmaf(t, t, ss);
     }
     if (!wn) return;
     const float inv_x = 1.0f / sqrtf(block_sum(ss, red) / (float)H + eps);
     TH* hr = h + r * H;
-    for (int i = threadIdx.x; i < H; i += blockDim.x) store_f32(hr + i, rowbuf[i] * inv_x * wn[i]);
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it) {
+        const int i = it * blockDim.x + threadIdx.x;
+        if (i < H) store_f32(hr + i, v[it] * inv_x * wnv[it]);
+    }
 }
 
 LLOGOS_EXPORT int llogos_sandwich_norm(float* x, const void* a, int a_dtype, int parts, long long part_stride, const float* wb,
                                        const float* wn, void* h, int h_dtype, float eps, int T, int H, hipStream_t stream) {
-    if (T <= 0 || H <= 0 || parts < 1 || (size_t)H * sizeof(float) > 65536) return LLOGOS_BAD_ARGUMENT;
-    const int threads = H >= 2048 ? 512 : (H >= 512 ? 256 : 128);
-    const size_t smem = (size_t)H * sizeof(float);
-#define SN(TA, TH) sandwich_norm_kernel<TA, TH><<<T, threads, smem, stream>>>(x, (const TA*)a, parts, (size_t)part_stride, wb, wn, (TH*)h, eps, H)
-    if (a_dtype == DT_F32 && h_dtype == DT_F32) SN(float, float);
-    else if (a_dtype == DT_F32 && h_dtype == DT_BF16) SN(float, bf16_t);
-    else if (a_dtype == DT_BF16 && h_dtype == DT_F32) SN(bf16_t, float);
-    else if (a_dtype == DT_BF16 && h_dtype == DT_BF16) SN(bf16_t, bf16_t);
+    if (T <= 0 || H <= 0 || parts < 1 || H > 16384) return LLOGOS_BAD_ARGUMENT;
+    // elements a thread: 1 for few rows (all of a row's loads in flight at once), up to 4 for many; blocks of up to 1024
+    int items = T >= 256 ? 4 : 1;
+    while ((H + items - 1) / items > 1024) items *= 2;
+    if (items > 16) return LLOGOS_BAD_ARGUMENT;
+    int threads = (H + items - 1) / items;
+    threads = (threads + kWave - 1) / kWave * kWave;
+#define SN(TA, TH, IT) sandwich_norm_kernel<TA, TH, IT><<<T, threads, 0, stream>>>(x, (const TA*)a, parts, (size_t)part_stride, wb, wn, (TH*)h, eps, H)
+#define SNI(TA, TH) do { if (items == 1) SN(TA, TH, 1); else if (items == 2) SN(TA, TH, 2); else if (items == 4) SN(TA, TH, 4); \
+                         else if (items == 8) SN(TA, TH, 8); else SN(TA, TH, 16); } while (0)
+    if (a_dtype == DT_F32 && h_dtype == DT_F32) SNI(float, float);
+    else if (a_dtype == DT_F32 && h_dtype == DT_BF16) SNI(float, bf16_t);
+    else if (a_dtype == DT_BF16 && h_dtype == DT_F32) SNI(bf16_t, float);
+    else if (a_dtype == DT_BF16 && h_dtype == DT_BF16) SNI(bf16_t, bf16_t);
     else return LLOGOS_BAD_ARGUMENT;
+#undef SNI
 #undef SN
     return LLOGOS_LAUNCH_CHECK();
 }

@@ -522,7 +522,7 @@ def latent_attention_mfma(ctx, q: torch.Tensor, k_pool: torch.Tensor, v_pool: to
         n_tiles = T * (-(-n_heads // 16))
         pages = max(1, min(table.shape[1], -(-ctx.max_context // PAGE_TOKENS)))
         want = max(1, (4 * compute_units()) // max(1, n_tiles))          # blocks of one wave's work: a few a compute unit
-        pps = max(1, -(-pages // min(pages, want)))
+        pps = max(1, -(-pages // min(pages, want, 16)))                  # (the merge kernel takes up to 16 parts)
         splits = -(-pages // pps)
         cu = None
         if splits > 1:
@@ -542,15 +542,23 @@ def latent_attention_mfma(ctx, q: torch.Tensor, k_pool: torch.Tensor, v_pool: to
     return out
 
 
-def head_products(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+def head_products(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_kn: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out[t, h, :N] = w[h] . a[t, h, :K] for every head h: a [T, H, >= K] and out [T, H, >= N] may be
-    views with their own row and head strides; w [H, N, K] is dense."""
+    views with their own row and head strides; w [H, N, K] is dense.  w_kn [H, K, N]: the same matrices
+    k-major, which steps of up to 16 rows stream instead (a kernel whose threads own an output each)."""
     _need(a.is_cuda and w.is_cuda and out.is_cuda and w.is_contiguous(), "head_products: device tensors, dense w")
     _need(a.dim() == 3 and out.dim() == 3 and w.dim() == 3, "head_products: a [T, H, K], w [H, N, K], out [T, H, N]")
     T, H, K = a.shape
     N = w.shape[1]
     _need(w.shape == (H, N, K) and out.shape == (T, H, N), "head_products: shapes do not fit")
     _need(a.stride(2) == 1 and out.stride(2) == 1, "head_products: unit inner strides")
+    if w_kn is not None and 0 < T <= 16:
+        _need(w_kn.is_cuda and w_kn.is_contiguous() and w_kn.shape == (H, K, N) and w_kn.dtype == w.dtype, "head_products: w_kn must be [H, K, N] like w")
+        code = _lib().llogos_head_products_few(_p(out), _dt(out), out.stride(0), out.stride(1), _p(a), _dt(a), a.stride(0), a.stride(1),
+                                               _p(w_kn), _dt(w_kn), T, H, N, K, _stream())
+        if code != -2:
+            _check(code, "head_products_few")
+            return out
     if T:
         _check(_lib().llogos_head_products(_p(out), _dt(out), out.stride(0), out.stride(1), _p(a), _dt(a), a.stride(0), a.stride(1),
                                            _p(w), _dt(w), T, H, N, K, _stream()), "head_products")

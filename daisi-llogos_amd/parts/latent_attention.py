@@ -46,7 +46,7 @@ class LatentAttention(Mixer):
         self.uq = Linear([prefix + "uq"], self.q_rank, [H * (self.dim + self.rot_dim)], suffix=suffix)
         self.dkv = Linear([prefix + "dkv"], hidden, [self.kv_rank + self.rot_dim], suffix=suffix)
         self.o = Linear([prefix + "o"], H * self.v_dim, [hidden], suffix=suffix)
-        self.uk_t = self.uv = self.q_norm_w = self.c_norm_w = self.sink = None
+        self.uk_t = self.uv = self.uk_kn = self.uv_kn = self.q_norm_w = self.c_norm_w = self.sink = None
 
     def _linears(self) -> List[Linear]:
         return [self.dq, self.uq, self.dkv, self.o]
@@ -84,6 +84,9 @@ class LatentAttention(Mixer):
         # per head the transposed key matrix [rank, dim]: a query's unrotated part times it is the query in the latent's space
         self.uk_t = uk.view(H, self.dim, self.kv_rank).transpose(1, 2).contiguous()
         self.uv = get(self.prefix + "uv").to(device=rt.device, dtype=rt.dtype).view(H, self.v_dim, self.kv_rank).contiguous()
+        # the same two sets of matrices k-major, for steps of few rows (a few MB a layer)
+        self.uk_kn = uk.view(H, self.dim, self.kv_rank).contiguous()
+        self.uv_kn = self.uv.transpose(1, 2).contiguous()
         if self.position is not None and getattr(self.position, "inv_freq", None) is None:
             self.position.bind(get, rt)
 
@@ -102,7 +105,7 @@ class LatentAttention(Mixer):
         qa = torch.empty((T, H, self.row), dtype=self.rt.dtype, device=h.device)
         K.latent_prepare(ctx, kv, q, qa, self.c_norm_w, self.eps, cs, cache.k_pool, cache.v_pool, cache.table, H, self.dim, self.rot_dim,
                          self.position.rot if self.position is not None else 0, self.kv_rank)
-        K.head_products(q.view(T, H, self.dim + self.rot_dim)[:, :, :self.dim], self.uk_t, qa[:, :, :self.kv_rank])
+        K.head_products(q.view(T, H, self.dim + self.rot_dim)[:, :, :self.dim], self.uk_t, qa[:, :, :self.kv_rank], self.uk_kn)
         mark(ctx, "rotation")
         lat = None
         if cache.v_pool is not None:
@@ -112,7 +115,7 @@ class LatentAttention(Mixer):
                                       self.scale, v_dim=self.kv_rank, head_sink=self.sink)
         mark(ctx, "attention")
         a = torch.empty((T, H, self.v_dim), dtype=self.rt.dtype, device=h.device)
-        K.head_products(lat.view(T, H, self.kv_rank), self.uv, a)
+        K.head_products(lat.view(T, H, self.kv_rank), self.uv, a, self.uv_kn)
         out = self.o.product(a.view(T, H * self.v_dim), f32_ok=True)
         mark(ctx, "o")
         return out
