@@ -20,16 +20,17 @@ from .pages import PAGE_TOKENS, CacheError, CacheFull, GroupPages, SlotAllocator
 
 
 class KVGroup:
-    def __init__(self, spec: KVSpec, entries: List[int], n_pages: int, rt: Optional[Runtime]):
+    def __init__(self, spec: KVSpec, entries: List[int], n_pages: int, rt: Optional[Runtime], spare: int = 0):
         self.spec = spec
         self.entries = entries                       # units that own storage here
         self.pages = GroupPages(n_pages, spec.window, spec.sinks)
         self.k = self.v = None
         if rt is not None:
             # a kv head's part of a page is PAGE_TOKENS * head size elements in the matrix cores'
-            # operand order (pages.key_offset, pages.value_offset); one page more than the pool
-            # hands out: the page of padding rows (Cache.pad_page)
-            shape = (len(entries), n_pages + 1, spec.n_kv_heads, PAGE_TOKENS * spec.head_dim)
+            # operand order (pages.key_offset, pages.value_offset); `spare` pages that the pool may
+            # come to hand out (Cache.spare_page_per_slot), and one page more: the page of padding
+            # rows (Cache.pad_page)
+            shape = (len(entries), n_pages + spare + 1, spec.n_kv_heads, PAGE_TOKENS * spec.head_dim)
             self.k = torch.zeros(shape, dtype=rt.dtype, device=rt.device)
             if spec.values:                  # (a latent cache has key rows only)
                 self.v = torch.zeros(shape, dtype=rt.dtype, device=rt.device)
@@ -46,9 +47,16 @@ class Cache:
 
     def __init__(self, needs: Sequence[Tuple[Optional[KVSpec], Optional[StateSpec]]],
                  reads_from: Sequence[Optional[int]], max_tokens: int, rt: Optional[Runtime],
-                 n_slots: int = 64):
+                 n_slots: int = 64, spare_page_per_slot: bool = False):
+        """spare_page_per_slot: max_tokens counts tokens, but a sequence holds whole pages, so several live
+        sequences can need up to a page each more than their tokens fill.  With this option every sequence
+        that is live beside another brings one page of its own to every pool (up to the first number of
+        slots; the pages' memory is set aside from the start), so that a caller who counted tokens is never
+        refused for the pages' rounding, while one sequence alone still gets max_tokens and no more."""
         self.rt = rt
         self.n_pages = max(1, pages_for(max_tokens))
+        self.spare = n_slots if spare_page_per_slot else 0        # pages set aside beyond n_pages
+        self.granted = 0                                          # of those, handed to the pools so far
         self.slots = SlotAllocator(n_slots)
         self.lengths: Dict[int, int] = {}
         self.groups: List[KVGroup] = []
@@ -59,7 +67,7 @@ class Cache:
                 by_spec.setdefault(kv, []).append(e)
         for spec, entries in by_spec.items():
             g = len(self.groups)
-            self.groups.append(KVGroup(spec, entries, self.n_pages, rt))
+            self.groups.append(KVGroup(spec, entries, self.n_pages, rt, self.spare))
             for i, e in enumerate(entries):
                 self.entry_group[e] = (g, i)
         for e, src in enumerate(reads_from):
@@ -80,6 +88,10 @@ class Cache:
             self._grow_slots(self.slots.n_slots * 2)
         slot = self.slots.alloc()
         self.lengths[slot] = 0
+        if self.granted < self.spare and len(self.lengths) > self.granted + 1:
+            for g in self.groups:                    # a sequence beside others: its page for the rounding
+                g.pages.pool.grow(1)
+            self.granted += 1
         for g in self.groups:
             g.pages.open(slot)
         for st in self.states:
@@ -111,7 +123,7 @@ class Cache:
 
     @property
     def pad_page(self) -> int:
-        return self.n_pages
+        return self.n_pages + self.spare
 
     def length(self, slot: int) -> int:
         self.slots.check(slot)

@@ -65,6 +65,12 @@ class PagePool:
     def free_count(self) -> int:
         return len(self._free)
 
+    def grow(self, n: int) -> None:
+        """n more pages, with the ids that follow the present ones."""
+        self._free = list(range(self.n_pages + n - 1, self.n_pages - 1, -1)) + self._free
+        self._held += [False] * n
+        self.n_pages += n
+
     def take(self, n: int) -> List[int]:
         if n > len(self._free):
             raise CacheFull(f"{n} pages wanted, {len(self._free)} of {self.n_pages} free")

@@ -92,7 +92,8 @@ class Engine:
     """A bound model with its cache.  `step` is the only way tokens reach the model."""
 
     def __init__(self, model: Model, rt: Runtime, max_tokens: int, n_slots: int = 64, config=None,
-                 use_graphs: Optional[bool] = None, max_seq: Optional[int] = None, architecture: str = ""):
+                 use_graphs: Optional[bool] = None, max_seq: Optional[int] = None, architecture: str = "",
+                 spare_page_per_slot: bool = False):
         self.model, self.rt, self.config = model, rt, config
         self.architecture = architecture or type(model).__name__      # the registry name the model was built under
         # The longest a sequence may become: the caller's limit (the reference's --max-context,
@@ -105,7 +106,7 @@ class Engine:
         if use_graphs is None:
             use_graphs = os.environ.get("LLOGOS_GRAPHS", "1") != "0"
         self.graphs = GraphCache(self) if (use_graphs and graph_ok) else None
-        self.cache = Cache(model.cache_needs(), model.cache_reads(), max_tokens, rt, n_slots)
+        self.cache = Cache(model.cache_needs(), model.cache_reads(), max_tokens, rt, n_slots, spare_page_per_slot)
         self.vocab_size = model.spec.vocab_size
         self.steps_run = 0
 
@@ -114,7 +115,7 @@ class Engine:
     def from_folder(cls, folder: str, dtype: Union[str, torch.dtype] = "bfloat16", max_tokens: int = 4096,
                     n_slots: int = 64, device: Union[str, torch.device] = "cuda:0",
                     use_graphs: Optional[bool] = None, max_seq: Optional[int] = None,
-                    pack_weights: Optional[bool] = None, **spec_options) -> "Engine":
+                    pack_weights: Optional[bool] = None, spare_page_per_slot: bool = False, **spec_options) -> "Engine":
         """config.json chooses the model class through the registry; model.safetensors is
         checked against what the model needs before any tensor is read.  pack_weights: None
         gives as many matrices a packed copy as the GPU's memory allows (packed_weight_budget)."""
@@ -134,7 +135,7 @@ class Engine:
                 torch.cuda.synchronize()
         finally:
             ckpt.close()
-        return cls(model, rt, max_tokens, n_slots, config, use_graphs, max_seq, arch.name)
+        return cls(model, rt, max_tokens, n_slots, config, use_graphs, max_seq, arch.name, spare_page_per_slot)
 
     @classmethod
     def from_config(cls, config: dict, seed: int = 0, dtype: Union[str, torch.dtype] = "bfloat16",

@@ -72,12 +72,11 @@ def main(argv=None) -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--out", required=True, help="folder for <step>.f32 files")
     ap.add_argument("--max-tokens", type=int, required=True,
-                    help="most tokens live requests hold at any time (each rounded up to 64); sizes the cache")
+                    help="most tokens live requests hold at any time; sizes the cache (a lone request may hold that many, "
+                         "rounded up to a page of 64; requests that are live together get a page each for the rounding)")
     args = ap.parse_args(argv)
-    # a request holds whole pages: one page more for each of the slots the engine starts with covers every
-    # request's last, partly filled page whatever way the caller counted
-    from ..cache.pages import PAGE_TOKENS
-    n_slots = 64
-    engine = Engine.from_folder(args.model, dtype=args.dtype, max_tokens=args.max_tokens + n_slots * PAGE_TOKENS, n_slots=n_slots)
+    # --max-tokens counts tokens and a request holds whole pages: every request that is live beside another
+    # brings a page of its own for its last, partly filled one (Cache: spare_page_per_slot)
+    engine = Engine.from_folder(args.model, dtype=args.dtype, max_tokens=args.max_tokens, spare_page_per_slot=True)
     replay(engine, sys.stdin, args.out)
     return 0

@@ -397,6 +397,7 @@ def wkv_scan(ctx, r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, d: torch.Te
 
 SCAN_COLUMN_BLOCKS = 0       # 0: chosen by the step; 1, 2, 4, ... force the number of blocks a head (tests)
 SCAN_SEGMENTS = 0            # 0: chosen by the step; 1, 2, 3, ... force the number of segments of a prompt (tests)
+SCAN_ROWS = 0                # 0: chosen by the step; 4 or 16 force the rows of the state a thread (tests)
 
 
 def scan_plan(batch: int, n_heads: int, dim: int, longest: Optional[int], n_cus: Optional[int] = None) -> Tuple[int, int, int]:
@@ -421,7 +422,7 @@ def scan_plan(batch: int, n_heads: int, dim: int, longest: Optional[int], n_cus:
         n_seg = SCAN_SEGMENTS
     if SCAN_COLUMN_BLOCKS and longest is not None:
         return 4, SCAN_COLUMN_BLOCKS, n_seg
-    if wide and waves16 * n_seg >= 2 * simds:
+    if SCAN_ROWS == 16 or (wide and waves16 * n_seg >= 2 * simds and not SCAN_ROWS):
         return 16, 1, n_seg
     blocks, pairs = 1, batch * n_heads * n_seg
     if longest is not None and longest >= 64:

@@ -101,6 +101,29 @@ def test_a_cache_without_a_device_counts_the_units(tmp_path):
     assert cache.free_pages() == [4]
 
 
+def test_sequences_that_are_live_together_bring_a_page_each_for_the_rounding():
+    m = _model(nc.NIP_B)
+    cache = L.Cache(m.cache_needs(), m.cache_reads(), 128, None, n_slots=4, spare_page_per_slot=True)
+    a = cache.alloc_slot()
+    assert cache.free_pages() == [2]                     # one sequence alone: what the tokens need and no more
+    with pytest.raises(L.CacheFull):
+        cache.reserve([a], [129])
+    b, c = cache.alloc_slot(), cache.alloc_slot()
+    assert cache.free_pages() == [4] and cache.pad_page == 2 + 4
+    cache.reserve([a, b, c], [70, 30, 28])               # 128 tokens in 2 + 1 + 1 pages
+    cache.commit([a, b, c], [70, 30, 28])
+    assert cache.free_pages() == [0]
+    cache.free_slot(b)
+    d = cache.alloc_slot()                               # three live again: nothing more is granted
+    assert cache.free_pages() == [1]
+    for s in (a, c, d):
+        cache.free_slot(s)
+    assert cache.free_pages() == [4]
+    plain = L.Cache(m.cache_needs(), m.cache_reads(), 128, None, n_slots=4)
+    plain.alloc_slot(), plain.alloc_slot()
+    assert plain.free_pages() == [2] and plain.pad_page == 2
+
+
 def test_yarn_frequencies_by_hand():
     # 8 rotated dimensions, base 100: f = 1, 100^-0.25, 100^-0.5, 100^-0.75
     f = rope.inverse_frequencies(8, 100.0)

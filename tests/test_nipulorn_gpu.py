@@ -118,12 +118,17 @@ def test_activations(kind):
 @pytest.mark.parametrize("heads,dim,hidden,rank,blocks", [(2, 40, 56, 6, 0), (1, 64, 64, 16, 0), (3, 24, 100, 5, 0), (2, 72, 48, 8, 0),
                                                           (5, 8, 64, 3, 0), (1, 128, 96, 4, 0), (1, 64, 64, 16, 4), (2, 40, 56, 6, 2),
                                                           (1, 128, 96, 4, 8), (3, 24, 100, 5, 3), (1, 64, 64, 16, -2), (2, 40, 56, 6, -3),
-                                                          (5, 8, 64, 3, -5), (1, 128, 96, 4, -2)])
+                                                          (5, 8, 64, 3, -5), (1, 128, 96, 4, -2), (1, 64, 64, 16, 16), (2, 48, 56, 6, 16),
+                                                          (3, 24, 100, 5, 16), (5, 8, 64, 3, 16), (1, 128, 96, 4, 16), (2, 40, 56, 6, -16)])
 def test_the_recurrent_mixer_alone_in_pieces(dtype, heads, dim, hidden, rank, blocks, monkeypatch):
     """blocks > 0: a head's state columns shared out over that many blocks in steps of several tokens, as
     long prompts of few sequences run, with the head norm in a kernel of its own.  blocks < 0: the steps of
     several tokens cut into that many segments that run side by side (more segments than some steps have
-    chunks: segments beyond a sequence's end), their states chained afterwards."""
+    chunks: segments beyond a sequence's end), their states chained afterwards.
+    blocks 16 and -16: 16 rows of the state a thread, as steps of many sequences run, whole and in 3 segments."""
+    if abs(blocks) == 16:
+        monkeypatch.setattr(K, "SCAN_ROWS", 16)
+        blocks = 0 if blocks > 0 else -3
     monkeypatch.setattr(K, "SCAN_COLUMN_BLOCKS", max(blocks, 0))
     monkeypatch.setattr(K, "SCAN_SEGMENTS", max(-blocks, 0))
     rng = np.random.default_rng(heads * dim)
