@@ -6,9 +6,9 @@
     score_h(i, j) = (q_h,plain(i) . k_h(j) + q_h,rot(i) . k_rot(j)) * scale,   j <= i
     weights = exp(score) / (sum_j exp(score) + exp(sink_h))
 
-Only c and the rotated key part are cached: one row [c | k_rot] a token, for all heads, and no
-values.  The scores are taken in the latent's space, q_h,plain . W_uk,h c = (W_uk,h^T q_h,plain) . c,
-so a head's query becomes [W_uk,h^T q_h,plain | q_h,rot] against the cached row, the weighted sum runs
+The cache holds one row [c | k_rot] a token, which serves every head, and no values of its own.
+The scores are taken in the latent's space, q_h,plain . W_uk,h c = (W_uk,h^T q_h,plain) . c, so a
+head's query becomes [W_uk,h^T q_h,plain | q_h,rot] against the cached row, the weighted sum runs
 over latents, and W_uv,h is applied to that sum."""
 from __future__ import annotations
 

@@ -18,7 +18,7 @@ class RMSNorm(Norm):
 
     def __init__(self, name: str, width: int, eps: float, offset: float = 0.0, suffix: str = ".weight"):
         """offset: the stored tensor is the weight less this number (1 for checkpoints that keep
-        their norm weights around zero); the sum is made once, in float32, when the tensor is bound.
+        their norm weights as the distance from one); the sum is made once, in float32, when the tensor is bound.
         suffix: what the tensor's name has behind `name`."""
         self.name = name
         self.width = width

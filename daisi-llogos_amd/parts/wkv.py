@@ -1,5 +1,5 @@
-"""A recurrent mixer with a matrix state per head (RWKV-style time mixing with a decay that
-depends on the token).
+"""A recurrent mixer with a matrix state per head (time mixing in the manner of RWKV, the decay
+made from the token).
 
 With h' the row before h (zeros before a sequence's first token), each of r, k, v, g, w reads its
 own mix m_s = h + (h' - h) * mu_s.  Then

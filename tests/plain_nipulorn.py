@@ -33,7 +33,7 @@ def root_mean_square_scale(x: np.ndarray, eps: float) -> np.ndarray:
 
 
 def offset_norm(x: np.ndarray, w: np.ndarray, eps: float) -> np.ndarray:
-    """RMS norm whose weight is stored around zero: the scale is 1 + w."""
+    """RMS norm whose stored weight w is an offset: the scale is 1 + w."""
     return root_mean_square_scale(x, eps) * (1.0 + np.asarray(w, dtype=np.float64))
 
 

@@ -229,7 +229,7 @@ def test_the_feed_forward_alone(dtype):
         assert np.abs(got - want[:n]).max() <= PART_TOL[dtype] * max(1.0, np.abs(want).max())
 
 
-def test_a_norm_with_a_weight_stored_around_zero():
+def test_a_norm_whose_stored_weight_is_an_offset_from_one():
     rng = np.random.default_rng(8)
     norm = P.RMSNorm("n", 50, 1e-5, offset=1.0, suffix="")
     plain = _bind(norm, rng, "float32")
