@@ -381,3 +381,24 @@ def test_the_trace_runner_on_a_model_of_the_design(tmp_path, dtype):
     for i in range(3):
         H.close(read(1 + i), np.concatenate([pa[70 + i:71 + i], pb[9 + i:10 + i]]), dtype, f"step {1 + i}")
     H.close(read(4), pa[74:75], dtype, "step 4")
+
+
+def test_the_command_line_on_a_model_of_the_design(tmp_path):
+    """`random` writes a model folder from a configuration file; generation from token ids prints what the
+    plain loop generates; --bench prints its block."""
+    name = "nip_b"
+    cfg_file = tmp_path / "config.json"
+    cfg_file.write_text(json.dumps(nc.ALL[name]))
+    out = tmp_path / "model"
+    run = lambda *args: subprocess.run([sys.executable, "-m", "daisi-llogos_amd", *args], capture_output=True, text=True, timeout=600, cwd=ROOT)
+    p = run("random", "--config", str(cfg_file), "--output-dir", str(out), "--seed", "4")
+    assert p.returncode == 0, p.stderr[-2000:]
+    cfg, w = pn.load_folder(str(out))
+    prompt = list(H.tokens(name, 11, 21))
+    p = run("--model", str(out), "--prompt", " ".join(map(str, prompt)), "-n", "6", "-t", "0", "--repeat-penalty", "1.0",
+            "--dtype", "float32", "--max-context", "64")
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert [int(t) for t in p.stdout.split()] == pn.generate_greedy(cfg, w, prompt, 6)
+    p = run("--model", str(out), "--bench", "--batch", "2", "-n", "8", "--prompt-len", "20", "--max-context", "64")
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert "decode" in (p.stdout + p.stderr)
