@@ -32,11 +32,11 @@ class KVGroup:
             # rows (Cache.pad_page)
             shape = (len(entries), n_pages + spare + 1, spec.n_kv_heads, PAGE_TOKENS * spec.head_dim)
             self.k = torch.zeros(shape, dtype=rt.dtype, device=rt.device)
-            if spec.values:                  # (a latent cache has key rows only)
-                self.v = torch.zeros(shape, dtype=rt.dtype, device=rt.device)
+            if spec.values:                  # (a latent cache has key rows only; values may be wider or narrower than keys)
+                self.v = torch.zeros(shape[:3] + (PAGE_TOKENS * spec.value_dim,), dtype=rt.dtype, device=rt.device)
 
     def bytes(self) -> int:
-        return 0 if self.k is None else (2 if self.v is not None else 1) * self.k.numel() * self.k.element_size()
+        return 0 if self.k is None else (self.k.numel() + (self.v.numel() if self.v is not None else 0)) * self.k.element_size()
 
 
 class Cache:
@@ -144,7 +144,8 @@ class Cache:
         if self.rt is None:
             return 0
         elt = torch.empty((), dtype=self.rt.dtype).element_size()
-        return sum((2 if g.spec.values else 1) * len(g.entries) * g.spec.n_kv_heads * g.spec.head_dim * elt for g in self.groups)
+        return sum(len(g.entries) * g.spec.n_kv_heads * (g.spec.head_dim + (g.spec.value_dim if g.spec.values else 0)) * elt
+                   for g in self.groups)
 
     # ---- a step's storage ----------------------------------------------------------
     def reserve(self, slot_ids: Sequence[int], new_lens: Sequence[int]) -> None:

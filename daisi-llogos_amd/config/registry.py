@@ -64,3 +64,12 @@ def _nipulorn() -> None:
 
 
 _nipulorn()
+
+
+def _zogurax() -> None:
+    from ..models.zogurax import zogurax_spec
+    from .zogurax_config import ZoguraxConfig
+    register_architecture("Zogurax", ZoguraxConfig.from_dict, zogurax_spec)
+
+
+_zogurax()

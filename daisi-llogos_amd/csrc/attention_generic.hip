@@ -7,7 +7,13 @@
 // Two options serve mixers whose cache differs from keys and values of one size:
 //   v_dim < head_dim with no value pool: a value is the first v_dim dimensions of its key row;
 //   head_sink [n_heads]: the softmax's denominator also holds exp(head_sink[h]), a learned score
-//   without a key or a value (the running maximum and sum start from it).
+//   without a key or a value (the running maximum and sum start from it); a sink of score 0 is the
+//   softmax with one added to its denominator.
+// Three more serve attention whose heads are shaped otherwise:
+//   v_page_dim: the value pool's pages hold rows of that many dimensions (values wider or narrower
+//   than keys; k_page_dim likewise is the key pages' row, which may be wider than head_dim);
+//   softcap > 0: a score s becomes softcap * tanh(s / softcap) before the softmax;
+//   gate [T, gate_stride]: head h's output is multiplied by sigmoid(gate[t, h]).
 // (reference: gated_attention / batched_gated_attention,
 //  Daisi.Llogos.Cuda/kernels/composite_ops.cu:275-387, 396-512: kv head = head / group,
 //  scale after the dot, tiles of 256 keys, running max and sum; the sigmoid gate of that
@@ -23,7 +29,8 @@ __global__ __launch_bounds__(256) void attn_generic_kernel(
         const T* __restrict__ k_pool, const T* __restrict__ v_pool, PagedKV cache,
         const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
         int n_heads, int group, int head_dim, float scale, int window, int sinks,
-        int v_dim, const float* __restrict__ head_sink) {
+        int v_dim, const float* __restrict__ head_sink, int v_page_dim, float softcap,
+        const float* __restrict__ gate, int gate_stride) {
     extern __shared__ float smem[];
     float* qf = smem;                    // [head_dim]
     float* p_lds = smem + head_dim;      // [kTileKeys]
@@ -49,8 +56,9 @@ __global__ __launch_bounds__(256) void attn_generic_kernel(
             const T* kpage = k_pool + paged_base(cache, seq, kvh, j);
             float dot = 0.f;
             for (int d = 0; d < head_dim; ++d)
-                dot = fmaf(qf[d], load_f32(kpage + page_key_offset(j % kPageTokens, d, head_dim)), dot);
+                dot = fmaf(qf[d], load_f32(kpage + page_key_offset(j % kPageTokens, d, cache.head_dim)), dot);
             s = dot * scale;
+            if (softcap > 0.f) s = softcap * tanhf(s / softcap);
         }
         const float tile_max = block_max(s, red);
         if (tile_max == -INFINITY) continue;
@@ -71,8 +79,8 @@ __global__ __launch_bounds__(256) void attn_generic_kernel(
                     if (pj != 0.f) {
                         const size_t base = paged_base(cache, seq, kvh, j0 + jj);
                         const int tk = (j0 + jj) % kPageTokens;
-                        a = fmaf(pj, v_pool ? load_f32(v_pool + base + page_value_offset(tk, d))
-                                            : load_f32(k_pool + base + page_key_offset(tk, d, head_dim)), a);
+                        a = fmaf(pj, v_pool ? load_f32(v_pool + base / cache.head_dim * v_page_dim + page_value_offset(tk, d))
+                                            : load_f32(k_pool + base + page_key_offset(tk, d, cache.head_dim)), a);
                     }
                 }
                 acc[r] = a;
@@ -81,7 +89,8 @@ __global__ __launch_bounds__(256) void attn_generic_kernel(
         l_run = l_run * corr + tile_sum;
         m_run = m_new;
     }
-    const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
+    float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
+    if (gate) inv *= 1.0f / (1.0f + expf(-gate[(size_t)t * gate_stride + h]));
     T* orow = out + ((size_t)t * n_heads + h) * v_dim;
 #pragma unroll
     for (int r = 0; r < kMaxHeadDimGeneric / 256; ++r) {
@@ -96,22 +105,26 @@ LLOGOS_EXPORT int llogos_attention_generic(void* out, const void* q, int dtype, 
                                            const int* tok_seq, const int* tok_pos,
                                            int T, int n_heads, int n_kv_heads, int head_dim,
                                            float scale, int window, int sinks, int v_dim, const float* head_sink,
+                                           int k_page_dim, int v_page_dim, float softcap, const float* gate, int gate_stride,
                                            hipStream_t stream) {
-    if (v_dim <= 0 || v_dim > head_dim || (!v_pool && !k_pool)) return LLOGOS_BAD_ARGUMENT;
+    if (k_page_dim <= 0) k_page_dim = head_dim;
+    if (v_page_dim <= 0) v_page_dim = k_page_dim;
+    if (v_dim <= 0 || v_dim > kMaxHeadDimGeneric || v_dim > (v_pool ? v_page_dim : head_dim) || !k_pool) return LLOGOS_BAD_ARGUMENT;
+    if (k_page_dim < head_dim || (k_page_dim % 8) || (v_page_dim % 16) || softcap < 0.f || (gate && gate_stride < n_heads)) return LLOGOS_BAD_ARGUMENT;
     if (T <= 0 || n_heads <= 0 || n_kv_heads <= 0 || n_heads % n_kv_heads != 0) return LLOGOS_BAD_ARGUMENT;
     if (head_dim <= 0 || head_dim > kMaxHeadDimGeneric || window < 0 || sinks < 0) return LLOGOS_BAD_ARGUMENT;
-    PagedKV cache{table, table_stride, n_kv_heads, head_dim};
+    PagedKV cache{table, table_stride, n_kv_heads, k_page_dim};
     dim3 grid(T, n_heads);
     const size_t smem = (size_t)(head_dim + kTileKeys + 16) * sizeof(float);
     const int group = n_heads / n_kv_heads;
     if (dtype == DT_F32)
         attn_generic_kernel<float><<<grid, 256, smem, stream>>>(
             (float*)out, (const float*)q, q_stride, (const float*)k_pool, (const float*)v_pool, cache,
-            tok_seq, tok_pos, n_heads, group, head_dim, scale, window, sinks, v_dim, head_sink);
+            tok_seq, tok_pos, n_heads, group, head_dim, scale, window, sinks, v_dim, head_sink, v_page_dim, softcap, gate, gate_stride);
     else if (dtype == DT_BF16)
         attn_generic_kernel<bf16_t><<<grid, 256, smem, stream>>>(
             (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, cache,
-            tok_seq, tok_pos, n_heads, group, head_dim, scale, window, sinks, v_dim, head_sink);
+            tok_seq, tok_pos, n_heads, group, head_dim, scale, window, sinks, v_dim, head_sink, v_page_dim, softcap, gate, gate_stride);
     else
         return LLOGOS_BAD_ARGUMENT;
     return LLOGOS_LAUNCH_CHECK();

@@ -40,6 +40,61 @@ LLOGOS_EXPORT int llogos_embed(float* out, const void* table, int table_dtype, c
     return LLOGOS_LAUNCH_CHECK();
 }
 
+// x[t, 2i] += sin(pos[t] * base^(-2i / W)), x[t, 2i + 1] += cos of the same angle: a position
+// vector of sines and cosines added to the embedding rows.  The frequency, the angle and its sine
+// and cosine are taken in double, as the rotary table's are.
+__global__ void add_sinusoid_kernel(float* __restrict__ x, const int* __restrict__ pos, int T, int W, double base) {
+    const int t = blockIdx.x;
+    const double p = (double)pos[t];
+    const int pairs = (W + 1) / 2;
+    for (int i = threadIdx.x; i < pairs; i += blockDim.x) {
+        const double a = p * exp(-log(base) * (2.0 * (double)i / (double)W));
+        float* o = x + (size_t)t * W + 2 * i;
+        o[0] += (float)sin(a);
+        if (2 * i + 1 < W) o[1] += (float)cos(a);
+    }
+}
+
+LLOGOS_EXPORT int llogos_add_sinusoid(float* x, const int* pos, int T, int W, double base, hipStream_t stream) {
+    if (T <= 0 || W <= 0 || !(base > 0.0)) return LLOGOS_BAD_ARGUMENT;
+    add_sinusoid_kernel<<<T, 128, 0, stream>>>(x, pos, T, W, base);
+    return LLOGOS_LAUNCH_CHECK();
+}
+
+// out[t] = [a[t] + delta[t] | b[t]] in out's type: two float32 streams side by side as one input row of
+// a product.  delta is optional and may come in parts; with write_back the sum also goes back to a.
+template <typename TO>
+__global__ void concat_rows_kernel(TO* __restrict__ out, float* __restrict__ a, const float* __restrict__ delta, int parts,
+                                   size_t part_stride, const float* __restrict__ b, int Wa, int Wb, int write_back) {
+    const int t = blockIdx.x;
+    TO* o = out + (size_t)t * (Wa + Wb);
+    for (int i = threadIdx.x; i < Wa + Wb; i += blockDim.x) {
+        float v;
+        if (i < Wa) {
+            v = a[(size_t)t * Wa + i];
+            if (delta) {
+                for (int q = 0; q < parts; ++q) v += delta[q * part_stride + (size_t)t * Wa + i];
+                if (write_back) a[(size_t)t * Wa + i] = v;
+            }
+        } else {
+            v = b[(size_t)t * Wb + (i - Wa)];
+        }
+        store_f32(o + i, v);
+    }
+}
+
+LLOGOS_EXPORT int llogos_concat_rows(void* out, int out_dtype, float* a, const float* delta, int parts, long long part_stride,
+                                     const float* b, int T, int Wa, int Wb, int write_back, hipStream_t stream) {
+    if (T <= 0 || Wa <= 0 || Wb <= 0 || parts < 1) return LLOGOS_BAD_ARGUMENT;
+    if (out_dtype == DT_F32)
+        concat_rows_kernel<float><<<T, 256, 0, stream>>>((float*)out, a, delta, parts, (size_t)part_stride, b, Wa, Wb, write_back);
+    else if (out_dtype == DT_BF16)
+        concat_rows_kernel<bf16_t><<<T, 256, 0, stream>>>((bf16_t*)out, a, delta, parts, (size_t)part_stride, b, Wa, Wb, write_back);
+    else
+        return LLOGOS_BAD_ARGUMENT;
+    return LLOGOS_LAUNCH_CHECK();
+}
+
 // x = x * scale, then, with cap > 0, x = cap * tanh(x / cap): scaled and soft-capped logits
 __global__ void scale_softcap_kernel(float* __restrict__ x, long long n, float scale, float cap) {
     const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;

@@ -1,0 +1,94 @@
+// From a token's projected row [q | k | v] to the attention's inputs, for attention without a
+// rotation: optional biases, an optional RMS norm over the whole of q and over the whole of k (all
+// heads at once, one weight a channel), an optional factor on the query that grows with the
+// logarithm of its position's block number, then q to a plain row and k and v to the cache's pages.
+//
+//   q' = rmsnorm_all(q + bq) * wq * (1 + coef * ln(floor((pos + 1) / every) + 1))
+//   k' = rmsnorm_all(k + bk) * wk                   -> key page of (sequence, position), head by head
+//   v' = v + bv                                     -> value page
+//
+// Keys have head_dim dimensions a head and values v_dim; their pages hold rows of k_page_dim and
+// v_page_dim (each the size rounded up to the pages' step).  The row comes as float32, maybe in
+// parts of a product split along k; norms, logarithm and factor are 32-bit.  One block a token.
+#include "common.h"
+
+template <typename T>
+__global__ __launch_bounds__(256) void qkv_prepare_kernel(
+        const float* __restrict__ qkv, int parts, size_t part_stride, int row_stride, const float* __restrict__ bias,
+        T* __restrict__ q_out, int n_heads, int n_kv_heads, int head_dim, int v_dim, int k_page_dim, int v_page_dim,
+        const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w, float eps, float temp_coef, int temp_every,
+        T* __restrict__ k_pool, T* __restrict__ v_pool, const int* __restrict__ table, int table_stride,
+        const int* __restrict__ tok_seq, const int* __restrict__ tok_pos) {
+    __shared__ float red[16];
+    const int t = blockIdx.x, tid = threadIdx.x;
+    const int Wq = n_heads * head_dim, Wk = n_kv_heads * head_dim, Wv = n_kv_heads * v_dim;
+    const float* row = qkv + (size_t)t * row_stride;
+    auto value = [&](int c) {
+        float v = row[c];
+        for (int p = 1; p < parts; ++p) v += row[p * part_stride + c];
+        if (bias) v += bias[c];
+        return v;
+    };
+    const int seq = tok_seq[t], pos = tok_pos[t];
+
+    float q_scale = 1.f, k_scale = 1.f;
+    if (q_norm_w) {
+        float ss = 0.f;
+        for (int c = tid; c < Wq; c += blockDim.x) { const float v = value(c); ss = fmaf(v, v, ss); }
+        q_scale = 1.0f / sqrtf(block_sum(ss, red) / (float)Wq + eps);
+    }
+    if (k_norm_w && Wk > 0) {
+        float ss = 0.f;
+        for (int c = tid; c < Wk; c += blockDim.x) { const float v = value(Wq + c); ss = fmaf(v, v, ss); }
+        k_scale = 1.0f / sqrtf(block_sum(ss, red) / (float)Wk + eps);
+    }
+    float temp = 1.f;
+    if (temp_coef != 0.f) temp = 1.0f + temp_coef * logf((float)((pos + 1) / temp_every + 1));
+
+    T* qo = q_out + (size_t)t * Wq;
+    for (int c = tid; c < Wq; c += blockDim.x) {
+        float v = value(c);
+        if (q_norm_w) v = v * q_scale * q_norm_w[c];
+        store_f32(qo + c, v * temp);
+    }
+    if (n_kv_heads <= 0) return;
+    const int page = table[(size_t)seq * table_stride + pos / kPageTokens];
+    const int in_page = pos % kPageTokens;
+    T* kp = k_pool + (size_t)page * n_kv_heads * kPageTokens * k_page_dim;
+    for (int c = tid; c < Wk; c += blockDim.x) {
+        float v = value(Wq + c);
+        if (k_norm_w) v = v * k_scale * k_norm_w[c];
+        const int g = c / head_dim, d = c % head_dim;
+        store_f32(kp + (size_t)g * kPageTokens * k_page_dim + page_key_offset(in_page, d, k_page_dim), v);
+    }
+    T* vp = v_pool + (size_t)page * n_kv_heads * kPageTokens * v_page_dim;
+    for (int c = tid; c < Wv; c += blockDim.x) {
+        const int g = c / v_dim, d = c % v_dim;
+        store_f32(vp + (size_t)g * kPageTokens * v_page_dim + page_value_offset(in_page, d), value(Wq + Wk + c));
+    }
+}
+
+// qkv: float32 rows [T, row_stride] (row_stride >= the three widths together), `parts` of them
+// part_stride apart; bias float32 [Wq + Wk + Wv] or null; q_norm_w [Wq], k_norm_w [Wk] or null.
+// n_kv_heads 0: the keys and values of these positions are another run's; only q is made.
+LLOGOS_EXPORT int llogos_qkv_prepare(const float* qkv, int parts, long long part_stride, int row_stride, const float* bias,
+                                     void* q_out, int dtype, int n_heads, int n_kv_heads, int head_dim, int v_dim,
+                                     int k_page_dim, int v_page_dim, const float* q_norm_w, const float* k_norm_w, float eps,
+                                     float temp_coef, int temp_every, void* k_pool, void* v_pool, const int* table,
+                                     int table_stride, const int* tok_seq, const int* tok_pos, int T, hipStream_t stream) {
+    if (T <= 0 || n_heads <= 0 || n_kv_heads < 0 || head_dim <= 0 || v_dim <= 0 || parts < 1) return LLOGOS_BAD_ARGUMENT;
+    if (temp_coef != 0.f && temp_every < 1) return LLOGOS_BAD_ARGUMENT;
+    if (n_kv_heads > 0) {
+        if (!k_pool || !v_pool || !table) return LLOGOS_BAD_ARGUMENT;
+        if (k_page_dim < head_dim || v_page_dim < v_dim || (k_page_dim % 8) || (v_page_dim % 16)) return LLOGOS_BAD_ARGUMENT;
+    }
+    if (row_stride < n_heads * head_dim + n_kv_heads * (head_dim + v_dim)) return LLOGOS_BAD_ARGUMENT;
+#define PREP(T_) qkv_prepare_kernel<T_><<<T, 256, 0, stream>>>(qkv, parts, (size_t)part_stride, row_stride, bias, (T_*)q_out, \
+        n_heads, n_kv_heads, head_dim, v_dim, k_page_dim, v_page_dim, q_norm_w, k_norm_w, eps, temp_coef, temp_every, \
+        (T_*)k_pool, (T_*)v_pool, table, table_stride, tok_seq, tok_pos)
+    if (dtype == DT_F32) PREP(float);
+    else if (dtype == DT_BF16) PREP(bf16_t);
+    else return LLOGOS_BAD_ARGUMENT;
+#undef PREP
+    return LLOGOS_LAUNCH_CHECK();
+}

@@ -6,7 +6,8 @@
 #include "common.h"
 
 // ---------------------------------------------------------------- short causal convolution
-// out[t, c] = h[t, c] + sum_j w[c, j] * h_(t - taps + 1 + j)[c]   (w[c, taps - 1] multiplies token t)
+// out[t, c] = [h[t, c] +] sum_j w[c, j] * h_(t - taps + 1 + j)[c]   (w[c, taps - 1] multiplies token t;
+// the input itself is added when add_input is set; rows of h lie ldh values apart)
 // Rows before the step's first token of a sequence come from the sequence's state
 // [taps - 1, W], whose row i holds the input at position (length - (taps - 1) + i); positions
 // before 0 count as zero.  cu (token offset of each sequence in the step) may be null: then
@@ -18,27 +19,27 @@ template <typename TO>
 __global__ void causal_conv_kernel(TO* __restrict__ out, const float* __restrict__ h, const float* __restrict__ w,
                                    float* __restrict__ state, const int* __restrict__ slots,
                                    const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
-                                   const int* __restrict__ cu, int W, int taps, int update_state) {
+                                   const int* __restrict__ cu, int W, int ldh, int taps, int update_state, int add_input) {
     const int t = blockIdx.x;
     const int seq = tok_seq[t], pos = tok_pos[t];
     const int before = cu ? t - cu[seq] : 0;                 // tokens of this sequence earlier in the step
     float* st = state + (size_t)slots[seq] * (taps - 1) * W;
     for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < W; c += gridDim.y * blockDim.x) {
         const float* wc = w + (size_t)c * taps;
-        const float x0 = h[(size_t)t * W + c];
+        const float x0 = h[(size_t)t * ldh + c];
         float acc = x0 * wc[taps - 1];
         float old[kMaxTaps];
 #pragma unroll
         for (int j = 1; j < kMaxTaps; ++j) {
             if (j < taps) {
                 float v = 0.f;
-                if (j <= before) v = h[(size_t)(t - j) * W + c];
+                if (j <= before) v = h[(size_t)(t - j) * ldh + c];
                 else if (pos - j >= 0) v = st[(size_t)(taps - 1 + before - j) * W + c];
                 old[j] = v;
                 acc = fmaf(wc[taps - 1 - j], v, acc);
             }
         }
-        store_f32(out + (size_t)t * W + c, x0 + acc);
+        store_f32(out + (size_t)t * W + c, add_input ? x0 + acc : acc);
         if (update_state) {                                  // one token a sequence: row i <- row i + 1, last <- this token
 #pragma unroll
             for (int j = 1; j < kMaxTaps; ++j)
@@ -51,7 +52,7 @@ __global__ void causal_conv_kernel(TO* __restrict__ out, const float* __restrict
 // from this step's rows or from the old state.  A thread owns a channel of a sequence and
 // reads all it needs before it writes.
 __global__ void conv_state_kernel(const float* __restrict__ h, float* __restrict__ state, const int* __restrict__ slots,
-                                  const int* __restrict__ cu, int W, int taps) {
+                                  const int* __restrict__ cu, int W, int ldh, int taps) {
     const int seq = blockIdx.x;
     const int first = cu[seq], count = cu[seq + 1] - first;
     float* st = state + (size_t)slots[seq] * (taps - 1) * W;
@@ -61,7 +62,7 @@ __global__ void conv_state_kernel(const float* __restrict__ h, float* __restrict
         for (int i = 0; i < kMaxTaps - 1; ++i) {
             if (i < taps - 1) {
                 const int back = taps - 1 - i;               // this row is the input `back` tokens before the new end
-                keep[i] = back <= count ? h[(size_t)(first + count - back) * W + c] : st[(size_t)(i + count) * W + c];
+                keep[i] = back <= count ? h[(size_t)(first + count - back) * ldh + c] : st[(size_t)(i + count) * W + c];
             }
         }
 #pragma unroll
@@ -72,20 +73,20 @@ __global__ void conv_state_kernel(const float* __restrict__ h, float* __restrict
 
 LLOGOS_EXPORT int llogos_causal_conv(void* out, int out_dtype, const float* h, const float* w, float* state,
                                      const int* slots, const int* tok_seq, const int* tok_pos, const int* cu,
-                                     int T, int B, int W, int taps, hipStream_t stream) {
-    if (T <= 0 || B <= 0 || W <= 0 || taps < 1 || taps > kMaxTaps) return LLOGOS_BAD_ARGUMENT;
+                                     int T, int B, int W, int ldh, int taps, int add_input, hipStream_t stream) {
+    if (T <= 0 || B <= 0 || W <= 0 || ldh < W || taps < 1 || taps > kMaxTaps) return LLOGOS_BAD_ARGUMENT;
     if (!cu && T != B) return LLOGOS_BAD_ARGUMENT;
     const int threads = 256;
     const int by = (W + threads - 1) / threads;
     dim3 grid(T, by);
     const int fused = cu ? 0 : 1;
     if (out_dtype == DT_F32)
-        causal_conv_kernel<float><<<grid, threads, 0, stream>>>((float*)out, h, w, state, slots, tok_seq, tok_pos, cu, W, taps, fused);
+        causal_conv_kernel<float><<<grid, threads, 0, stream>>>((float*)out, h, w, state, slots, tok_seq, tok_pos, cu, W, ldh, taps, fused, add_input);
     else if (out_dtype == DT_BF16)
-        causal_conv_kernel<bf16_t><<<grid, threads, 0, stream>>>((bf16_t*)out, h, w, state, slots, tok_seq, tok_pos, cu, W, taps, fused);
+        causal_conv_kernel<bf16_t><<<grid, threads, 0, stream>>>((bf16_t*)out, h, w, state, slots, tok_seq, tok_pos, cu, W, ldh, taps, fused, add_input);
     else
         return LLOGOS_BAD_ARGUMENT;
-    if (cu && taps > 1) conv_state_kernel<<<dim3(B, by), threads, 0, stream>>>(h, state, slots, cu, W, taps);
+    if (cu && taps > 1) conv_state_kernel<<<dim3(B, by), threads, 0, stream>>>(h, state, slots, cu, W, ldh, taps);
     return LLOGOS_LAUNCH_CHECK();
 }
 
@@ -543,32 +544,36 @@ LLOGOS_EXPORT int llogos_sandwich_norm(float* x, const void* a, int a_dtype, int
 //   0 tanh;  1 silu;  2 gelu (tanh form);
 //   3 the piecewise xIELU with a = softplus(p), b = 1/2 + softplus(q):
 //       z > 0: a z^2 + z / 2;   z <= 0: b (exp(z) - 1 - z) + z / 2
-enum { ACT_TANH = 0, ACT_SILU = 1, ACT_GELU_TANH = 2, ACT_XIELU = 3 };
+//   4 the square of relu: max(z, 0)^2
+enum { ACT_TANH = 0, ACT_SILU = 1, ACT_GELU_TANH = 2, ACT_XIELU = 3, ACT_RELU2 = 4 };
 
 __device__ __forceinline__ float activate(float z, int kind, float a, float b) {
     switch (kind) {
         case ACT_TANH: return tanhf(z);
         case ACT_SILU: return z / (1.0f + expf(-z));
         case ACT_GELU_TANH: return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+        case ACT_RELU2: { const float r = fmaxf(z, 0.f); return r * r; }
         default: return z > 0.f ? fmaf(a * z, z, 0.5f * z) : fmaf(b, expm1f(z) - z, 0.5f * z);
     }
 }
 
 template <typename TO, typename TI>
 __global__ void activation_kernel(TO* __restrict__ out, const TI* __restrict__ in, int parts, size_t part_stride,
-                                  size_t n, int kind, float a, float b) {
+                                  size_t n, int kind, float a, float b, int cols, int ld_in) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
-    float z = load_f32(in + i);
-    for (int q = 1; q < parts; ++q) z += load_f32(in + q * part_stride + i);
+    // cols > 0: the input's rows lie ld_in values apart and their first `cols` values are taken (out is dense)
+    const size_t src = cols > 0 ? (i / cols) * (size_t)ld_in + i % cols : i;
+    float z = load_f32(in + src);
+    for (int q = 1; q < parts; ++q) z += load_f32(in + q * part_stride + src);
     store_f32(out + i, activate(z, kind, a, b));
 }
 
 LLOGOS_EXPORT int llogos_activation(void* out, int out_dtype, const void* in, int in_dtype, int parts, long long part_stride,
-                                    long long n, int kind, float a, float b, hipStream_t stream) {
-    if (n <= 0 || parts < 1 || kind < 0 || kind > ACT_XIELU) return LLOGOS_BAD_ARGUMENT;
+                                    long long n, int kind, float a, float b, int cols, int ld_in, hipStream_t stream) {
+    if (n <= 0 || parts < 1 || kind < 0 || kind > ACT_RELU2 || cols < 0 || (cols > 0 && ld_in < cols)) return LLOGOS_BAD_ARGUMENT;
     const unsigned blocks = (unsigned)((n + 255) / 256);
-#define ACT(TO, TI) activation_kernel<TO, TI><<<blocks, 256, 0, stream>>>((TO*)out, (const TI*)in, parts, (size_t)part_stride, (size_t)n, kind, a, b)
+#define ACT(TO, TI) activation_kernel<TO, TI><<<blocks, 256, 0, stream>>>((TO*)out, (const TI*)in, parts, (size_t)part_stride, (size_t)n, kind, a, b, cols, ld_in)
     if (out_dtype == DT_F32 && in_dtype == DT_F32) ACT(float, float);
     else if (out_dtype == DT_BF16 && in_dtype == DT_F32) ACT(bf16_t, float);
     else if (out_dtype == DT_BF16 && in_dtype == DT_BF16) ACT(bf16_t, bf16_t);

@@ -65,7 +65,8 @@ def packed_weight_budget(model: Model, dtype: torch.dtype, max_tokens: int, devi
             for d in spec.shape:
                 n *= int(d)
             elements += n
-    cache = max_tokens * sum((2 if kv.values else 1) * kv.n_kv_heads * kv.head_dim * element for kv, _ in model.cache_needs() if kv is not None)
+    cache = max_tokens * sum(kv.n_kv_heads * (kv.head_dim + (kv.value_dim if kv.values else 0)) * element
+                             for kv, _ in model.cache_needs() if kv is not None)
     with torch.cuda.device(device):
         free, total = torch.cuda.mem_get_info()
         free += torch.cuda.memory_reserved() - torch.cuda.memory_allocated()      # what torch holds but does not use

@@ -34,6 +34,9 @@ class ScheduleEntry:
     several); None gives the run a cache of its own."""
     layer: int
     cache_of: Optional[int] = None
+    # (index into ModelSpec.stream_parts, pass number): that part transforms the stream right before this
+    # run (the head of a pass through a run of layers that is gone through several times)
+    enter: Optional[Tuple[int, int]] = None
 
 
 @dataclass
@@ -51,6 +54,11 @@ class ModelSpec:
     embed_scale: float = 1.0       # the embedding rows are multiplied by this (1: a row copy)
     logit_scale: float = 1.0       # the logits are multiplied by this ...
     logit_softcap: float = 0.0     # ... and then, if > 0, bent to cap * tanh(logit / cap)
+    head_suffix: str = ".weight"   # what the head matrix's tensor name has behind head_name
+    position_vector: float = 0.0   # > 0: sines and cosines of the position at frequencies base^(-2i / width) join the embedding
+    # parts that stand between layers and transform the stream, named by schedule entries' `enter`:
+    # (registry, kind, parameters) triples like LayerSpec.more; forward(ctx, x, pending, x0, number) -> (x, pending)
+    stream_parts: List[object] = field(default_factory=list)
 
 
 _REGISTRIES = {"mixer": (MIXERS, "mixer"), "feed_forward": (FEED_FORWARDS, "feed-forward"), "norm": (NORMS, "norm"),
@@ -86,6 +94,7 @@ class Model:
         self.spec = spec
         self.layers = [build_layer(ls) for ls in spec.layers]
         self.final_norm = make(NORMS, "norm", spec.final_norm[0], **spec.final_norm[1])
+        self.stream_parts = [_make_part(t) for t in spec.stream_parts]
         self.schedule = list(spec.schedule) if spec.schedule is not None else \
             [ScheduleEntry(i) for i in range(len(self.layers))]
         self.entry_units: List[List[int]] = []               # schedule entry -> its units
@@ -93,11 +102,13 @@ class Model:
         for e in self.schedule:
             if not 0 <= e.layer < len(self.layers):
                 raise ValueError(f"a schedule entry names layer {e.layer}, the model has {len(self.layers)}")
+            if e.enter is not None and not 0 <= e.enter[0] < len(self.stream_parts):
+                raise ValueError(f"a schedule entry names stream part {e.enter[0]}, the model has {len(self.stream_parts)}")
             mixers = self.layers[e.layer].cache_parts()       # the mixers, and whatever else keeps state
             self.entry_units.append(list(range(len(self.unit_mixers), len(self.unit_mixers) + len(mixers))))
             self.unit_mixers += mixers
         self._check_schedule()
-        self.head = Linear([spec.head_name], spec.hidden_size, [spec.vocab_size])
+        self.head = Linear([spec.head_name], spec.hidden_size, [spec.vocab_size], suffix=spec.head_suffix)
         self.embed_table: Optional[torch.Tensor] = None
         self.rt: Optional[Runtime] = None
 
@@ -126,9 +137,11 @@ class Model:
         specs = [TensorSpec(s.embed_name, (s.vocab_size, s.hidden_size), "table")]
         for layer in self.layers:
             specs += layer.tensor_specs()
+        for part in self.stream_parts:
+            specs += part.tensor_specs()
         specs += self.final_norm.tensor_specs()
         if not s.tie_head:
-            specs.append(TensorSpec(s.head_name + ".weight", (s.vocab_size, s.hidden_size), "matrix"))
+            specs.append(TensorSpec(s.head_name + s.head_suffix, (s.vocab_size, s.hidden_size), "matrix"))
         return specs
 
     # ---- what the cache must hold ---------------------------------------------
@@ -156,6 +169,8 @@ class Model:
         self.embed_table = _to_device([get(self.spec.embed_name)], rt.dtype, rt.device)
         for layer in self.layers:
             layer.bind(get, rt)
+        for part in self.stream_parts:
+            part.bind(get, rt)
         self.final_norm.bind(get, rt)
         if self.spec.tie_head:
             self.head.bind_shared(self.embed_table, rt)      # one allocation serves both
@@ -180,11 +195,12 @@ class Model:
         """Bytes of weights a step reads once: every scheduled run of a layer, the final norm and
         the head (of the embedding table a step reads a row a token, which is not counted)."""
         runs = sum(self.layers[e.layer].weight_bytes() for e in self.schedule)
+        runs += sum(self.stream_parts[e.enter[0]].weight_bytes() for e in self.schedule if e.enter is not None)
         return runs + self.final_norm.weight_bytes() + self.head.weight_bytes()
 
     def packed_weight_bytes(self) -> int:
         """Bytes of device memory that the packed second copies of the matrices take (each layer once)."""
-        return sum(layer.packed_bytes() for layer in self.layers) + self.head.packed_bytes()
+        return sum(p.packed_bytes() for p in self.layers + self.stream_parts) + self.head.packed_bytes()
 
     def step_flops(self, lens: List[int], starts: Optional[List[int]] = None, wanted_rows: int = 0) -> float:
         """Floating-point operations of a step that brings lens[i] tokens to sequence i, which
@@ -194,6 +210,7 @@ class Model:
         starts = starts or [0] * len(lens)
         tokens = sum(lens)
         total = 2.0 * tokens * sum(self.layers[e.layer].matrix_elements() for e in self.schedule)
+        total += 2.0 * tokens * sum(self.stream_parts[e.enter[0]].matrix_elements() for e in self.schedule if e.enter is not None)
         pairs = sum(n * s + n * (n + 1) / 2.0 for n, s in zip(lens, starts))        # (query, visible key) pairs
         for m in self.unit_mixers:
             if hasattr(m, "n_heads") and hasattr(m, "head_dim"):
@@ -207,14 +224,24 @@ class Model:
         None when nothing is wanted."""
         s = self.spec
         x = K.embed(self.embed_table, ctx.ids, s.embed_scale)
+        if s.position_vector > 0.0:
+            K.add_sinusoid(x, ctx.tok_pos, s.position_vector)
         ctx.mark("embed")
         pending = None
         blocks = [self.layers[entry.layer] for entry in self.schedule]
+        # the embedding output, for stream parts that read it again; the stream itself is changed in place
+        x0 = x.clone() if any(e.enter is not None for e in self.schedule[1:]) else x
         for i, (block, units) in enumerate(zip(blocks, self.entry_units)):
+            enter = self.schedule[i].enter
+            if enter is not None:
+                x, pending = self.stream_parts[enter[0]].forward(ctx, x, pending, x0, enter[1])
+                ctx.mark("enter")
             if block.takes_next_norm:
                 # the norm that reads the stream after this block: the next block's first one, the final
                 # norm after the last (None: the next block has no such norm and takes `pending` as a tensor)
-                next_norm = blocks[i + 1].entry_norm() if i + 1 < len(blocks) else self.final_norm
+                # (a stream part in between takes the stream as it is: no norm's rows are prepared for it)
+                next_norm = (blocks[i + 1].entry_norm() if self.schedule[i + 1].enter is None else None) \
+                    if i + 1 < len(blocks) else self.final_norm
                 x, pending = block.forward(ctx, x, pending, [caches[u] for u in units], next_norm=next_norm)
             else:
                 x, pending = block.forward(ctx, x, pending, [caches[u] for u in units])

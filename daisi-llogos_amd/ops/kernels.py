@@ -163,6 +163,54 @@ def residual_add(x: torch.Tensor, delta: torch.Tensor) -> None:
            "residual_add")
 
 
+def layernorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
+              delta: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None, write_back: bool = True) -> torch.Tensor:
+    """(v - mean) / sqrt(variance + eps) * weight of the rows v = x + delta of the float32 stream x [T, H]
+    (delta [T, H] or partial sums [parts, T, H]; with write_back the sum goes back to x); `rows` picks rows."""
+    _dev(x, weight, delta, rows)
+    _i32(rows, "rows")
+    _need(x.dtype == torch.float32 and x.dim() == 2, "layernorm: the stream must be float32 [T, H]")
+    T, H = x.shape
+    _need(weight.dtype == torch.float32 and weight.shape == (H,), "layernorm: weight must be float32 [H]")
+    parts, part_stride = _parts(delta)
+    if delta is not None:
+        _need(tuple(delta.shape[-2:]) == (T, H), "layernorm: delta must be [T, H] or [parts, T, H]")
+        _need(parts == 1 or delta.dtype == torch.float32, "layernorm: parts must be float32")
+    R = T if rows is None else rows.numel()
+    out = torch.empty((R, H), dtype=out_dtype, device=x.device)
+    if R:
+        _check(_lib().llogos_layernorm(_p(out), _DT[out_dtype], _p(x), _p(delta), _dt(delta) if delta is not None else F32, parts,
+                                       ctypes.c_longlong(part_stride), _p(rows), _p(weight), ctypes.c_float(eps), R, H,
+                                       1 if write_back else 0, _stream()), "layernorm")
+    return out
+
+
+def add_sinusoid(x: torch.Tensor, positions: torch.Tensor, base: float = 10000.0) -> torch.Tensor:
+    """In place on float32 x [T, W]: x[t, 2i] += sin(p_t * base^(-2i / W)), x[t, 2i + 1] += cos of the same."""
+    _dev(x, positions)
+    _i32(positions, "positions")
+    _need(x.dtype == torch.float32 and x.dim() == 2 and positions.numel() == x.shape[0], "add_sinusoid: float32 [T, W] and T positions")
+    _check(_lib().llogos_add_sinusoid(_p(x), _p(positions), x.shape[0], x.shape[1], ctypes.c_double(base), _stream()), "add_sinusoid")
+    return x
+
+
+def concat_rows(a: torch.Tensor, b: torch.Tensor, out_dtype: torch.dtype, delta: Optional[torch.Tensor] = None,
+                write_back: bool = True) -> torch.Tensor:
+    """[a + delta | b] row by row in `out_dtype`: float32 a [T, Wa] and b [T, Wb]; delta float32 [T, Wa] or
+    partial sums [parts, T, Wa], added to a on the way (and written back to it)."""
+    _dev(a, b, delta)
+    _need(a.dtype == torch.float32 and b.dtype == torch.float32 and a.dim() == 2 and b.dim() == 2 and a.shape[0] == b.shape[0],
+          "concat_rows: two float32 tensors of as many rows")
+    parts, part_stride = _parts(delta)
+    if delta is not None:
+        _need(delta.dtype == torch.float32 and tuple(delta.shape[-2:]) == tuple(a.shape), "concat_rows: delta must be float32 like a")
+    T, Wa, Wb = a.shape[0], a.shape[1], b.shape[1]
+    out = torch.empty((T, Wa + Wb), dtype=out_dtype, device=a.device)
+    _check(_lib().llogos_concat_rows(_p(out), _DT[out_dtype], _p(a), _p(delta), parts, ctypes.c_longlong(part_stride), _p(b), T, Wa, Wb,
+                                     1 if write_back else 0, _stream()), "concat_rows")
+    return out
+
+
 def gemm_generic(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out_dtype: torch.dtype,
                  out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """a [M, K] . w [N, K]^T (+ bias) with plain 32-bit FMAs."""
@@ -241,31 +289,99 @@ def attention_generic(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_po
                       table: torch.Tensor, tok_seq: torch.Tensor, tok_pos: torch.Tensor,
                       n_heads: int, n_kv_heads: int, head_dim: int, scale: float,
                       window: int = 0, sinks: int = 0, v_dim: Optional[int] = None,
-                      head_sink: Optional[torch.Tensor] = None) -> torch.Tensor:
+                      head_sink: Optional[torch.Tensor] = None, softcap: float = 0.0,
+                      gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention of T query rows (row stride `q_stride` elements, heads first) over the
     paged cache; returns [T, n_heads * v_dim] in the cache's element type.  `v_pool` None:
     a value is the first `v_dim` dimensions of its key row.  `head_sink` float32 [n_heads]:
-    a learned score per head that joins the softmax's denominator without a key or a value."""
+    a learned score per head that joins the softmax's denominator without a key or a value.
+    With a value pool, values may have another width than keys (`v_dim`), and the pages' rows may be
+    wider than either (the pools' last dimension says so).  `softcap` > 0 bends every score to
+    softcap * tanh(score / softcap); `gate` float32 [T, >= n_heads] (a view of wider rows will do)
+    multiplies head h's output by sigmoid(gate[t, h])."""
     _dev(k_pool, v_pool, table, tok_seq, tok_pos)
     _i32(tok_seq, "tok_seq"); _i32(tok_pos, "tok_pos"); _i32(table, "table")
     T = tok_seq.numel()
     _need(q.is_cuda and q.dtype == k_pool.dtype, "attention: q and cache types differ")
     _need(n_heads % n_kv_heads == 0, "attention: heads must be a multiple of kv heads")
     _need(0 < head_dim <= GENERIC_MAX_HEAD_DIM, f"attention: head_dim {head_dim} not in 1..{GENERIC_MAX_HEAD_DIM}")
-    _check_pools(k_pool, v_pool, n_kv_heads, head_dim, "attention")
+    k_page_dim, v_page_dim = _page_dims(k_pool, v_pool, n_kv_heads, "attention")
+    _need(k_page_dim >= head_dim, "attention: the key pages' rows are narrower than a head")
     _need(q_stride >= n_heads * head_dim and q.numel() >= (T - 1) * q_stride + n_heads * head_dim,
           "attention: q too small")
     v_dim = head_dim if v_dim is None else int(v_dim)
-    _need(0 < v_dim <= head_dim, "attention: value width outside 1..head_dim")
+    _need(0 < v_dim <= (v_page_dim if v_pool is not None else head_dim) and v_dim <= GENERIC_MAX_HEAD_DIM,
+          "attention: value width outside what the pages hold")
     if head_sink is not None:
         _dev(head_sink)
         _need(head_sink.dtype == torch.float32 and head_sink.shape == (n_heads,), "attention: head_sink must be float32 [n_heads]")
+    gate_stride = 0
+    if gate is not None:
+        _need(gate.is_cuda and gate.dtype == torch.float32 and gate.dim() == 2 and gate.shape[0] == T and gate.shape[1] >= n_heads
+              and gate.stride(1) == 1, "attention: gate must be float32 [T, n_heads]")
+        gate_stride = gate.stride(0) if T > 1 else max(n_heads, gate.stride(0))
+    _need(softcap >= 0.0, "attention: softcap must not be negative")
     out = torch.empty((T, n_heads * v_dim), dtype=q.dtype, device=q.device)
     _check(_lib().llogos_attention_generic(
         _p(out), _p(q), _dt(q), q_stride, _p(k_pool), _p(v_pool), _p(table), table.stride(0),
         _p(tok_seq), _p(tok_pos), T, n_heads, n_kv_heads, head_dim, ctypes.c_float(scale),
-        window, sinks, v_dim, _p(head_sink), _stream()), "attention_generic")
+        window, sinks, v_dim, _p(head_sink), k_page_dim, v_page_dim, ctypes.c_float(softcap), _p(gate), gate_stride,
+        _stream()), "attention_generic")
     return out
+
+
+def _page_dims(k_pool: torch.Tensor, v_pool: Optional[torch.Tensor], n_kv_heads: int, who: str) -> Tuple[int, int]:
+    """(key row, value row) of the pools' pages, from their shapes [pages, kv_heads, PAGE_TOKENS * row]."""
+    _need(k_pool.dim() == 3 and k_pool.shape[1] == n_kv_heads and k_pool.shape[2] % (PAGE_TOKENS * 8) == 0 and k_pool.is_contiguous(),
+          f"{who}: key pool must be [pages, kv_heads, {PAGE_TOKENS} * row]")
+    kd = k_pool.shape[2] // PAGE_TOKENS
+    if v_pool is None:
+        return kd, kd
+    _need(v_pool.dim() == 3 and tuple(v_pool.shape[:2]) == tuple(k_pool.shape[:2]) and v_pool.shape[2] % (PAGE_TOKENS * 16) == 0
+          and v_pool.is_contiguous() and v_pool.dtype == k_pool.dtype,
+          f"{who}: value pool must be [pages, kv_heads, {PAGE_TOKENS} * row] like the key pool")
+    return kd, v_pool.shape[2] // PAGE_TOKENS
+
+
+def qkv_prepare(ctx, qkv: torch.Tensor, bias: Optional[torch.Tensor], out_dtype: torch.dtype, n_heads: int, n_kv_heads: int,
+                head_dim: int, v_dim: int, q_norm_w: Optional[torch.Tensor], k_norm_w: Optional[torch.Tensor], eps: float,
+                temp_coef: float, temp_every: int, k_pool: Optional[torch.Tensor], v_pool: Optional[torch.Tensor],
+                table: Optional[torch.Tensor], writes: bool = True) -> torch.Tensor:
+    """From projected rows [q | k | v | ...] (float32 [T, >= W] or partial sums [parts, T, >= W], plus `bias`
+    [W], W = n_heads * head_dim + n_kv_heads * (head_dim + v_dim)): an RMS norm over the whole of q and of
+    k where a weight is given ([n_heads * head_dim], [n_kv_heads * head_dim]), the query's factor
+    1 + temp_coef * ln(floor((pos + 1) / temp_every) + 1); q comes back [T, n_heads * head_dim] in
+    `out_dtype`, k and v go to their pages.  writes False: only q is made."""
+    _need(qkv.is_cuda and qkv.dtype == torch.float32 and qkv.stride(-1) == 1, "qkv_prepare: float32 rows on the GPU")
+    _dev(bias, q_norm_w, k_norm_w, table, ctx.tok_seq, ctx.tok_pos)
+    parts, part_stride = _parts(qkv)
+    T = qkv.shape[-2]
+    Wq, Wk, Wv = n_heads * head_dim, n_kv_heads * head_dim, n_kv_heads * v_dim
+    width = Wq + Wk + Wv
+    _need(qkv.shape[-1] >= width and T == ctx.n_tokens, f"qkv_prepare: rows of at least {width} values, one a token")
+    row_stride = qkv.stride(-2) if T > 1 else max(width, qkv.stride(-2))
+    if bias is not None:
+        _need(bias.dtype == torch.float32 and bias.numel() >= width, f"qkv_prepare: bias must be float32 [{width}]")
+    if q_norm_w is not None:
+        _need(q_norm_w.dtype == torch.float32 and q_norm_w.shape == (Wq,), f"qkv_prepare: q norm weight float32 [{Wq}]")
+    if k_norm_w is not None:
+        _need(k_norm_w.dtype == torch.float32 and k_norm_w.shape == (Wk,), f"qkv_prepare: k norm weight float32 [{Wk}]")
+    _need(temp_coef == 0.0 or temp_every >= 1, "qkv_prepare: the temperature's block must be at least one position")
+    kd = vd = 0
+    if writes:
+        _need(k_pool is not None and v_pool is not None and table is not None, "qkv_prepare: cache missing")
+        _i32(table, "table")
+        _need(k_pool.dtype == out_dtype, "qkv_prepare: cache type differs")
+        kd, vd = _page_dims(k_pool, v_pool, n_kv_heads, "qkv_prepare")
+        _need(kd >= head_dim and vd >= v_dim and table.dim() == 2, "qkv_prepare: pages narrower than the heads")
+    q_out = torch.empty((T, Wq), dtype=out_dtype, device=qkv.device)
+    _check(_lib().llogos_qkv_prepare(
+        _p(qkv), parts, ctypes.c_longlong(part_stride), row_stride, _p(bias), _p(q_out), _DT[out_dtype], n_heads,
+        n_kv_heads if writes else 0, head_dim, v_dim, kd, vd, _p(q_norm_w), _p(k_norm_w), ctypes.c_float(eps),
+        ctypes.c_float(temp_coef), int(temp_every), _p(k_pool) if writes else None, _p(v_pool) if writes else None,
+        _p(table) if writes else None, table.stride(0) if (writes and table is not None) else 0, _p(ctx.tok_seq), _p(ctx.tok_pos),
+        T, _stream()), "qkv_prepare")
+    return q_out
 
 
 def swiglu(gu: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
@@ -310,16 +426,18 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
 # parts with a fixed-size state per sequence
 # ----------------------------------------------------------------------------
 MAX_CONV_TAPS = 16
-ACTIVATIONS = {"tanh": 0, "silu": 1, "gelu_tanh": 2, "xielu": 3}
+ACTIVATIONS = {"tanh": 0, "silu": 1, "gelu_tanh": 2, "xielu": 3, "relu2": 4}
 
 
-def causal_conv(ctx, h: torch.Tensor, w: torch.Tensor, state: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
-    """h + conv(h) over time, channel by channel: h float32 [T, W] (the step's rows, one sequence
-    after the other), w float32 [W, taps] whose last tap multiplies the present token, state
-    float32 [slots, taps - 1, W]: a sequence's last taps - 1 inputs, read for the rows before the
-    step's first and brought up to date."""
-    _dev(h, w, state, ctx.slots, ctx.tok_seq, ctx.tok_pos, ctx.cu_dev)
-    _need(h.dtype == torch.float32 and h.dim() == 2, "causal_conv: h must be float32 [T, W]")
+def causal_conv(ctx, h: torch.Tensor, w: torch.Tensor, state: torch.Tensor, out_dtype: torch.dtype,
+                add_input: bool = True) -> torch.Tensor:
+    """h + conv(h) over time, channel by channel (conv(h) alone with add_input False): h float32 [T, W]
+    (the step's rows, one sequence after the other; it may be the first W columns of wider rows), w
+    float32 [W, taps] whose last tap multiplies the present token, state float32 [slots, taps - 1, W]: a
+    sequence's last taps - 1 inputs, read for the rows before the step's first and brought up to date."""
+    _need(h.is_cuda and h.dim() == 2 and h.stride(1) == 1, "causal_conv: h must be rows on the GPU")
+    _dev(w, state, ctx.slots, ctx.tok_seq, ctx.tok_pos, ctx.cu_dev)
+    _need(h.dtype == torch.float32, "causal_conv: h must be float32 [T, W]")
     T, W = h.shape
     _need(w.dtype == torch.float32 and w.dim() == 2 and w.shape[0] == W and 1 <= w.shape[1] <= MAX_CONV_TAPS,
           f"causal_conv: w must be float32 [W, taps] with at most {MAX_CONV_TAPS} taps")
@@ -330,7 +448,8 @@ def causal_conv(ctx, h: torch.Tensor, w: torch.Tensor, state: torch.Tensor, out_
     _need(ctx.cu_dev is not None or T == ctx.batch, "causal_conv: a step of several tokens a sequence needs the token offsets")
     out = torch.empty((T, W), dtype=out_dtype, device=h.device)
     _check(_lib().llogos_causal_conv(_p(out), _DT[out_dtype], _p(h), _p(w), _p(state), _p(ctx.slots), _p(ctx.tok_seq),
-                                     _p(ctx.tok_pos), _p(ctx.cu_dev), T, ctx.batch, W, taps, _stream()), "causal_conv")
+                                     _p(ctx.tok_pos), _p(ctx.cu_dev), T, ctx.batch, W, h.stride(0) if T > 1 else max(W, h.stride(0)),
+                                     taps, 1 if add_input else 0, _stream()), "causal_conv")
     return out
 
 
@@ -450,19 +569,92 @@ def sandwich_norm(x: torch.Tensor, a: torch.Tensor, post_w: torch.Tensor, next_w
     return h
 
 
-def activation(x: torch.Tensor, kind: str, out_dtype: torch.dtype, a: float = 0.0, b: float = 0.0) -> torch.Tensor:
+def activation(x: torch.Tensor, kind: str, out_dtype: torch.dtype, a: float = 0.0, b: float = 0.0,
+               cols: Optional[int] = None) -> torch.Tensor:
     """act(x) element by element; x [T, N] or float32 partial sums [parts, T, N] that are added first.
-    kinds: tanh, silu, gelu_tanh, xielu (z > 0: a z^2 + z / 2; z <= 0: b (exp(z) - 1 - z) + z / 2)."""
+    kinds: tanh, silu, gelu_tanh, xielu (z > 0: a z^2 + z / 2; z <= 0: b (exp(z) - 1 - z) + z / 2), relu2
+    (the square of max(z, 0)).  cols: only the first `cols` values of every row are taken (the result is
+    [T, cols]): a product whose rows hold something else behind them."""
     _dev(x)
     _need(kind in ACTIVATIONS, f"activation: unknown kind '{kind}'; known: {sorted(ACTIVATIONS)}")
     parts, part_stride = _parts(x)
     _need(parts == 1 or x.dtype == torch.float32, "activation: parts must be float32")
     T, N = x.shape[-2:]
-    out = torch.empty((T, N), dtype=out_dtype, device=x.device)
+    C = N if cols is None else int(cols)
+    _need(0 < C <= N, "activation: cols outside 1..N")
+    out = torch.empty((T, C), dtype=out_dtype, device=x.device)
     if out.numel():
         _check(_lib().llogos_activation(_p(out), _DT[out_dtype], _p(x), _dt(x), parts, ctypes.c_longlong(part_stride),
-                                        ctypes.c_longlong(T * N), ACTIVATIONS[kind], ctypes.c_float(a), ctypes.c_float(b), _stream()),
+                                        ctypes.c_longlong(T * C), ACTIVATIONS[kind], ctypes.c_float(a), ctypes.c_float(b),
+                                        0 if C == N else C, N, _stream()),
                "activation")
+    return out
+
+
+# ----------------------------------------------------------------------------
+# experts chosen by a table over token ids
+# ----------------------------------------------------------------------------
+MOE_MAX_EXPERTS = 1024
+
+
+def moe_route(ids: torch.Tensor, table: torch.Tensor, n_experts: int):
+    """(order, seg, where) int32 on the device: the step's (token, choice) pairs t * top + j sorted by
+    their expert table[ids[t], j], the experts' segments in that order (n_experts + 1 offsets) and each
+    pair's place in it."""
+    _dev(ids, table)
+    _i32(ids, "ids"); _i32(table, "table")
+    _need(ids.dim() == 1 and table.dim() == 2 and 0 < n_experts <= MOE_MAX_EXPERTS, f"moe_route: ids [T], table [V, top], at most {MOE_MAX_EXPERTS} experts")
+    T, top = ids.numel(), table.shape[1]
+    buf = torch.empty(2 * T * top + n_experts + 1, dtype=torch.int32, device=ids.device)
+    order, where, seg = buf[:T * top], buf[T * top:2 * T * top], buf[2 * T * top:]
+    _check(_lib().llogos_moe_route(_p(ids), _p(table), T, top, n_experts, _p(order), _p(seg), _p(where), _stream()), "moe_route")
+    return order, seg, where
+
+
+def moe_product(a: torch.Tensor, w: torch.Tensor, order: torch.Tensor, seg: torch.Tensor, top: int, gather: bool,
+                out_dtype: torch.dtype, relu2: bool = False, scale: float = 1.0) -> torch.Tensor:
+    """[P, N]: sorted row r, which belongs to the expert e whose segment holds it, is a_row(r) . w[e]^T, with
+    a_row(r) = a[order[r] // top] (gather: a holds the step's token rows) or a[r] (a is sorted already);
+    w [E, N, K]; relu2 squares max(., 0) in the epilogue, scale multiplies the result."""
+    _dev(a, w, order, seg)
+    _i32(order, "order"); _i32(seg, "seg")
+    _need(a.dim() == 2 and w.dim() == 3 and a.shape[1] == w.shape[2] and seg.numel() == w.shape[0] + 1, "moe_product: a [M, K], w [E, N, K]")
+    _need(a.dtype == w.dtype, "moe_product: rows and matrices of one type")
+    E, N, Kk = w.shape
+    P = order.numel()
+    _need(gather or a.shape[0] == P, "moe_product: sorted rows must be as many as pairs")
+    _need(not gather or a.shape[0] * top == P, "moe_product: token rows times choices must be the pairs")
+    out = torch.empty((P, N), dtype=out_dtype, device=a.device)
+    _check(_lib().llogos_moe_product(_p(out), _DT[out_dtype], _p(a), _dt(a), _p(w), _dt(w), _p(order), _p(seg), E, top,
+                                     1 if gather else 0, P, N, Kk, a.stride(0), 1 if relu2 else 0, ctypes.c_float(scale), _stream()),
+           "moe_product")
+    return out
+
+
+def moe_combine(y: torch.Tensor, where: torch.Tensor, top: int, shared: Optional[torch.Tensor] = None,
+                gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """float32 [T, W]: the mean of each token's pair rows y[where[t * top + j]], plus its shared row times
+    sigmoid(gate[t]).  shared float32 [T, W] or parts [parts, T, W]; gate a float32 column [T, 1] (a view of
+    one column of wider rows will do) or parts [parts, T, 1] of it."""
+    _dev(y, where)
+    _i32(where, "where")
+    _need(y.dtype == torch.float32 and y.dim() == 2 and where.numel() == y.shape[0] and y.shape[0] % top == 0, "moe_combine: y float32 [T * top, W]")
+    T, W = y.shape[0] // top, y.shape[1]
+    parts, part_stride = 1, 0
+    if shared is not None:
+        _dev(shared)
+        parts, part_stride = _parts(shared)
+        _need(shared.dtype == torch.float32 and tuple(shared.shape[-2:]) == (T, W), "moe_combine: shared rows float32 [T, W]")
+    g_parts, g_part_stride, g_stride = 1, 0, 1
+    if gate is not None:
+        _need(gate.is_cuda and gate.dtype == torch.float32 and gate.dim() in (2, 3) and tuple(gate.shape[-2:]) == (T, 1),
+              "moe_combine: gate float32 [T, 1]")
+        g_stride = gate.stride(-2) if T > 1 else 1
+        if gate.dim() == 3:
+            g_parts, g_part_stride = gate.shape[0], gate.stride(0)
+    out = torch.empty((T, W), dtype=torch.float32, device=y.device)
+    _check(_lib().llogos_moe_combine(_p(out), _p(y), _p(where), top, _p(shared), parts, ctypes.c_longlong(part_stride), _p(gate),
+                                     g_stride, g_parts, ctypes.c_longlong(g_part_stride), T, W, _stream()), "moe_combine")
     return out
 
 

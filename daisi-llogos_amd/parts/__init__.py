@@ -3,11 +3,14 @@ from .base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, OTHER_PARTS, POSITIONS,
                    Mixer, Norm, NormedRows, Part, PositionEncoding, Residual, Runtime, StateSpec, StepContext, TensorSpec, make,
                    register_block, register_feed_forward, register_mixer, register_norm, register_part, register_position)
 from .linear import Linear
-from .norm import RMSNorm
+from .norm import LayerNorm, RMSNorm
 from .rope import Rotary
 from .attention import Attention
 from .conv import CausalConv
 from .wkv import WKV
 from .latent_attention import LatentAttention
 from .mlp import ActivatedMLP, SwiGLU
-from .block import PreNormBlock, SandwichBlock
+from .capped_attention import CappedAttention
+from .moe import TableMoE
+from .loop import LoopEntry
+from .block import ParallelBlock, PreNormBlock, SandwichBlock

@@ -47,6 +47,11 @@ class KVSpec:
     window: int = 0
     sinks: int = 0
     values: bool = True     # False: no value pool; the mixer's values are part of its key rows (a latent cache)
+    v_dim: int = 0          # width of a value row in its pages when it is not head_dim (0: the same)
+
+    @property
+    def value_dim(self) -> int:
+        return self.v_dim or self.head_dim
 
 
 @dataclass(frozen=True)

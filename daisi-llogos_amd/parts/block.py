@@ -154,3 +154,49 @@ class SandwichBlock(Block):
         rows, delta = self._close(x, d, self.post_ffn_norm, next_norm, True)
         mark(ctx, "norm")
         return x, (delta if rows is None else NormedAhead(rows, next_norm))
+
+
+@register_block("parallel")
+class ParallelBlock(Block):
+    """One norm, and a mixer and a feed-forward that both read its output and both add to the stream:
+
+        h = norm(x);   x += mixer(h) + ffn(h)
+
+    The feed-forward may be absent.  The mixer's output joins the stream at once (through its closing
+    product where that can add itself, else by a sum kernel), the feed-forward's is handed on as `pending`;
+    without a feed-forward the mixer's output is."""
+
+    def __init__(self, mixer_norm: Norm, mixer: Mixer, ffn: Optional[FeedForward] = None):
+        self.mixer_norm, self.mixer, self.ffn = mixer_norm, mixer, ffn
+
+    def mixers(self) -> List[Mixer]:
+        return [self.mixer]
+
+    def feed_forwards(self) -> List[FeedForward]:
+        return [self.ffn] if self.ffn is not None else []
+
+    def parts(self) -> List[Part]:
+        return [p for p in (self.mixer_norm, self.mixer, self.ffn) if p is not None]
+
+    def entry_norm(self) -> Optional[Norm]:
+        return self.mixer_norm
+
+    def forward(self, ctx: StepContext, x: torch.Tensor, pending, caches):
+        from ..ops import kernels as K
+        cache = caches[0] if isinstance(caches, (list, tuple)) else caches
+        h = self.mixer_norm.forward(x, pending)
+        mark(ctx, "norm")
+        if self.mixer.adds_to_residual:
+            a = self.mixer.forward(ctx, h, cache, residual=Residual(x, None))
+        else:
+            a = self.mixer.forward(ctx, h, cache)
+        if isinstance(a, K.RowSquares):
+            a = None                                     # the mixer's closing product has added itself to x
+        mark(ctx, "mixer")
+        if self.ffn is None:
+            return x, a
+        if a is not None:
+            K.residual_add(x, K.sum_parts(a, None, torch.float32))
+        d = self.ffn.forward(ctx, h)
+        mark(ctx, "feed_forward")
+        return x, d

@@ -16,7 +16,7 @@ class Linear(Part):
     the output row is the concatenation of their outputs."""
 
     def __init__(self, names: Sequence[str], in_features: int, out_features: Sequence[int],
-                 bias: bool = False, suffix: str = ".weight", gated: bool = False):
+                 bias: bool = False, suffix: str = ".weight", gated: bool = False, bias_suffix: str = ".bias"):
         # gated: the two stacked matrices are a gate and an up projection whose product is only ever
         # wanted as silu(gate) * up; their packed copy then serves the product that makes that in its
         # epilogue (gated_product)
@@ -24,6 +24,7 @@ class Linear(Part):
             and out_features[0] % 16 == 0 and not bias
         self.names = list(names)
         self.suffix = suffix                             # what a matrix's tensor name has behind its name in `names`
+        self.bias_suffix = bias_suffix                   # and what its bias has there
         self.in_features = in_features
         self.out_features = list(out_features)
         self.has_bias = bias
@@ -40,7 +41,7 @@ class Linear(Part):
         for n, o in zip(self.names, self.out_features):
             specs.append(TensorSpec(n + self.suffix, (o, self.in_features), "matrix"))
             if self.has_bias:
-                specs.append(TensorSpec(n + ".bias", (o,), "bias"))
+                specs.append(TensorSpec(n + self.bias_suffix, (o,), "bias"))
         return specs
 
     def bind(self, get: Callable[[str], Optional[torch.Tensor]], rt: Runtime) -> None:
@@ -49,7 +50,7 @@ class Linear(Part):
         self.weight = _to_device(mats, rt.dtype, rt.device)
         self._pack(rt)
         if self.has_bias:
-            self.bias = _to_device([get(n + ".bias") for n in self.names], torch.float32, rt.device)
+            self.bias = _to_device([get(n + self.bias_suffix) for n in self.names], torch.float32, rt.device)
 
     def matrix_elements(self) -> int:
         return self.in_features * self.total_out

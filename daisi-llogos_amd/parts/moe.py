@@ -1,0 +1,96 @@
+"""A mixture of experts without a router: a table over token ids names each token's experts.
+
+    out_t = (1 / top) sum_j expert_(table[id_t, j])(h_t)  +  sigmoid(w_sg . h_t) * shared(h_t)
+    expert(h) = W_down act(W_up h)          (no biases; the shared expert has the same form)
+
+The table is an integer tensor [vocab, top] whose rows hold different experts.  The choice is made
+on the device from the step's ids, so single-token steps can be captured and replayed.  The
+experts' matrices are stacked ([experts, ff, width] and [experts, width, ff]); the (token, choice)
+pairs are sorted by expert and each expert's rows multiplied tile by tile."""
+from __future__ import annotations
+
+from typing import Callable, List, Optional
+
+import torch
+
+from ..ops import kernels as K
+from .base import FeedForward, Runtime, StepContext, TensorSpec, mark, register_feed_forward
+from .linear import Linear
+
+_EPILOGUES = ("relu2",)        # activations that the experts' product applies in its epilogue
+
+
+def _float32(product: torch.Tensor) -> torch.Tensor:
+    """A product as float32 (in parts or not), for consumers that read nothing else."""
+    return product if product.dtype == torch.float32 else K.sum_parts(product, None, torch.float32)
+
+
+@register_feed_forward("table_moe")
+class TableMoE(FeedForward):
+    graph_safe = True
+
+    def __init__(self, prefix: str, hidden: int, vocab: int, n_experts: int, top: int, intermediate: int,
+                 shared_intermediate: int = 0, activation: str = "relu2"):
+        if not 1 <= top <= n_experts <= K.MOE_MAX_EXPERTS:
+            raise ValueError(f"top {top} of {n_experts} experts: outside 1..experts..{K.MOE_MAX_EXPERTS}")
+        if activation not in _EPILOGUES:
+            raise ValueError(f"unknown expert activation '{activation}'; known: {list(_EPILOGUES)}")
+        self.prefix, self.hidden, self.vocab = prefix, int(hidden), int(vocab)
+        self.n_experts, self.top, self.intermediate = int(n_experts), int(top), int(intermediate)
+        self.shared_intermediate, self.activation = int(shared_intermediate), activation
+        self.table = self.up = self.down = None
+        self.shared_up = self.shared_down = None
+        if self.shared_intermediate:
+            # the gate's row rides behind the shared expert's up matrix: one product for both
+            self.shared_up = Linear([prefix + "shared.up", prefix + "shared.sg"], hidden, [self.shared_intermediate, 1], suffix="")
+            self.shared_down = Linear([prefix + "shared.down"], self.shared_intermediate, [hidden], suffix="")
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        p = self.prefix
+        specs = []
+        for e in range(self.n_experts):
+            specs += [TensorSpec(f"{p}e{e}.up", (self.intermediate, self.hidden), "matrix"),
+                      TensorSpec(f"{p}e{e}.down", (self.hidden, self.intermediate), "matrix")]
+        specs.append(TensorSpec(p + "table", (self.vocab, self.top), f"choices:{self.n_experts}"))
+        if self.shared_up is not None:
+            specs += self.shared_up.tensor_specs() + self.shared_down.tensor_specs()
+        return specs
+
+    def bind(self, get: Callable[[str], Optional[torch.Tensor]], rt: Runtime) -> None:
+        super().bind(get, rt)
+        p, E = self.prefix, self.n_experts
+        self.up = torch.empty((E, self.intermediate, self.hidden), dtype=rt.dtype, device=rt.device)
+        self.down = torch.empty((E, self.hidden, self.intermediate), dtype=rt.dtype, device=rt.device)
+        for e in range(E):
+            self.up[e].copy_(get(f"{p}e{e}.up"))
+            self.down[e].copy_(get(f"{p}e{e}.down"))
+        table = get(p + "table")
+        if table.dtype.is_floating_point:
+            raise ValueError(f"{p}table must hold integers")
+        table = table.to(torch.int64)
+        if table.numel() and (int(table.min()) < 0 or int(table.max()) >= E):
+            raise ValueError(f"{p}table names experts outside 0..{E - 1}")
+        self.table = table.to(device=rt.device, dtype=torch.int32).contiguous()
+        if self.shared_up is not None:
+            self.shared_up.bind(get, rt)
+            self.shared_down.bind(get, rt)
+
+    def matrix_elements(self) -> int:
+        """What a token is multiplied with: its `top` experts and the shared one."""
+        return super().matrix_elements() + 2 * self.top * self.intermediate * self.hidden
+
+    def forward(self, ctx: StepContext, h: torch.Tensor):
+        order, seg, where = K.moe_route(ctx.ids, self.table, self.n_experts)
+        act = K.moe_product(h, self.up, order, seg, self.top, True, self.rt.dtype, relu2=True)
+        y = K.moe_product(act, self.down, order, seg, self.top, False, torch.float32)
+        mark(ctx, "experts")
+        shared = gate = None
+        if self.shared_up is not None:
+            z = _float32(self.shared_up.product(h, f32_ok=True))             # [(parts,) T, ff + 1]
+            a = K.activation(z, self.activation, self.rt.dtype, cols=self.shared_intermediate)
+            shared = _float32(self.shared_down.product(a, f32_ok=True))
+            gate = z[..., self.shared_intermediate:]
+            mark(ctx, "shared")
+        out = K.moe_combine(y, where, self.top, shared, gate)
+        mark(ctx, "combine")
+        return out

@@ -1,4 +1,4 @@
-"""RMSNorm with the residual sum fused in.
+"""Norms with the residual sum fused in: RMSNorm, and a layer norm with a weight and no bias.
 out = v * rsqrt(mean(v^2) + eps) * w with v = x + delta; eps inside the root and the weight
 as it is (reference: Daisi.Llogos.Cpu/RmsNorm.cs:14-65; fused forms
 Daisi.Llogos/IComputeBackend.cs:417-466)."""
@@ -54,3 +54,27 @@ class RMSNorm(Norm):
 
     def row_weight(self) -> Optional[torch.Tensor]:
         return self.weight
+
+
+@register_norm("layernorm")
+class LayerNorm(Norm):
+    """out = (v - mean(v)) / sqrt(var(v) + eps) * w with v = x + delta, the variance being the mean of
+    the squared deviations; a weight and no bias.  It is no norm of the form `x * w * (a scale of the
+    row)`, so it has no row weight and takes tensors only."""
+
+    def __init__(self, name: str, width: int, eps: float, suffix: str = ".weight"):
+        self.name, self.width, self.eps, self.suffix = name, int(width), float(eps), suffix
+        self.weight: Optional[torch.Tensor] = None
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return [TensorSpec(self.name + self.suffix, (self.width,), "norm")]
+
+    def bind(self, get: Callable[[str], Optional[torch.Tensor]], rt: Runtime) -> None:
+        super().bind(get, rt)
+        self.weight = get(self.name + self.suffix).to(device=rt.device, dtype=torch.float32).contiguous()
+
+    def forward(self, x: torch.Tensor, delta=None, rows: Optional[torch.Tensor] = None,
+                write_back: bool = True, lazy: bool = False, out_dtype: Optional[torch.dtype] = None):
+        if isinstance(delta, (NormedAhead, K.RowSquares)):
+            delta = None               # whoever left that has completed the stream; its rows are another norm's
+        return K.layernorm(x, self.weight, self.eps, out_dtype or self.rt.dtype, delta=delta, rows=rows, write_back=write_back)

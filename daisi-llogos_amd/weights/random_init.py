@@ -67,6 +67,8 @@ def random_tensor(spec: TensorSpec, seed: int, dtype: torch.dtype, std: float = 
     their last bit between devices, which survives the rounding to `dtype` about once in 2^44
     elements for bfloat16: a model made on the GPU is the model written to a folder."""
     keys = _keys(seed, spec.name)
+    if spec.kind.startswith("choices:"):
+        return _choice_rows(spec, keys, device)
     n = 1
     for d in spec.shape:
         n *= int(d)
@@ -76,6 +78,23 @@ def random_tensor(spec: TensorSpec, seed: int, dtype: torch.dtype, std: float = 
         count = min(chunk, n - first)
         out[first:first + count] = _random_chunk(first, count, keys, spec.kind, std, device).to(dtype)
     return out.view(tuple(spec.shape))
+
+
+def is_integer_kind(kind: str) -> bool:
+    """Kinds of tensors that hold integers whatever type the model's numbers are stored in."""
+    return kind.startswith("choices:")
+
+
+def _choice_rows(spec: TensorSpec, keys: Tuple[int, int], device) -> torch.Tensor:
+    """int32 [rows, top] for the kind 'choices:<n>': every row names `top` different numbers below n,
+    a start drawn for the row and the numbers that follow it, around the end."""
+    n = int(spec.kind.split(":", 1)[1])
+    rows, top = (int(d) for d in spec.shape)
+    if top > n:
+        raise ValueError(f"{spec.name}: {top} different choices out of {n}")
+    idx = torch.arange(rows, dtype=torch.int64, device=device)
+    start = _mix32(_mix32((idx + keys[0]) & _MASK32) ^ keys[1]) % n
+    return ((start[:, None] + torch.arange(top, dtype=torch.int64, device=device)[None, :]) % n).to(torch.int32)
 
 
 def random_tensors(model: Model, seed: int, dtype: torch.dtype, std: float = 0.02,
@@ -103,6 +122,6 @@ def write_random_model(folder: str, config: dict, seed: int = 0, std: float = 0.
     os.makedirs(folder, exist_ok=True)
     with open(os.path.join(folder, "config.json"), "w") as fh:
         json.dump(config, fh, indent=2)
-    layout = [(s.name, tuple(s.shape), store) for s in model.tensor_specs()]
+    layout = [(s.name, tuple(s.shape), torch.int32 if is_integer_kind(s.kind) else store) for s in model.tensor_specs()]
     write_safetensors(os.path.join(folder, "model.safetensors"), random_tensors(model, seed, store, std, device), layout)
     return folder
