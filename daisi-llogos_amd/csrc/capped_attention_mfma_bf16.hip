@@ -1,0 +1,334 @@
+// bfloat16 attention on the matrix cores for heads whose keys and values have different widths,
+// whose scores may be bent through a tanh (s -> cap * tanh(s / cap)), whose softmax may carry a
+// sink of score 0 (one added to the denominator) and whose output may be gated head by head
+// (sigmoid of a logit a token and head).  No window: a query sees every key up to its own.
+//
+// Keys are rows of KP = 32 KS dimensions in their pages, values rows of VP = 16 VB; the pages are
+// in the matrix cores' operand order (common.h), so the page steps of attention_mfma.h serve:
+// one wave works on 16 columns and one page of 64 keys at a time.
+//   prefill: the columns are 16 consecutive tokens of a sequence for one query head; a block of 4
+//            waves takes a tile of 64 tokens; every wave walks the pages up to its last row.
+//   decode:  the columns are the query heads of one kv head; a block of 4 waves takes a run of
+//            pages of one (sequence, kv head), each wave every fourth of them; the waves' results
+//            are merged through LDS, and blocks along the context leave partial results
+//            (max, sum, output) for a small merge kernel.
+// The sink and the gate are applied where a row is finished (a block's own write, or the merge).
+#include "attention_mfma.h"
+
+// Softmax of one page with the score's scale and bend applied first, in place of softmax_page
+// (which folds a plain scale into its exponent).  y = bend(s * scale) * log2(e); the tanh is
+// 1 - 2 / (exp(2 x) + 1), with the hardware's exp2 and reciprocal.
+template <bool MASKED, int VP>
+__device__ __forceinline__ void softmax_page_bent(f32x4 (&s)[4], WaveState<VP>& st, float scale, float cap, int q_pos,
+                                                  int key0, bf16x8 (&pf)[2], float& corr) {
+    const int g = (threadIdx.x & (kWave - 1)) >> 4;
+    const float two_over_cap_log2 = cap > 0.f ? 2.0f * kLog2e / cap : 0.f;
+    float y[16];
+    float tile_max = -INFINITY;
+#pragma unroll
+    for (int rb = 0; rb < 4; ++rb)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            float x = s[rb][r] * scale;
+            if (cap > 0.f) {
+                const float t = __builtin_amdgcn_exp2f(x * two_over_cap_log2);
+                x = cap * (1.0f - 2.0f * __builtin_amdgcn_rcpf(t + 1.0f));
+            }
+            x *= kLog2e;
+            if (MASKED) {
+                const int key = key0 + g * 16 + rb * 4 + r;
+                if (!(q_pos >= 0 && key <= q_pos)) x = -INFINITY;
+            }
+            y[4 * rb + r] = x;
+            tile_max = fmaxf(tile_max, x);
+        }
+    tile_max = quad_max(tile_max);
+    const float m_new = fmaxf(st.m, tile_max);
+    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+    corr = __builtin_amdgcn_exp2f(st.m - m_use);
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        y[i] = __builtin_amdgcn_exp2f(y[i] - m_use);
+        sum += y[i];
+    }
+    sum = quad_sum(sum);
+    st.l = st.l * corr + sum;
+    st.m = m_new;
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        uint4 u;
+        u.x = pack_bf16(y[8 * t + 0], y[8 * t + 1]);
+        u.y = pack_bf16(y[8 * t + 2], y[8 * t + 3]);
+        u.z = pack_bf16(y[8 * t + 4], y[8 * t + 5]);
+        u.w = pack_bf16(y[8 * t + 6], y[8 * t + 7]);
+        pf[t] = __builtin_bit_cast(bf16x8, u);
+    }
+}
+
+template <int KP, int VP>
+__device__ __forceinline__ void attend_page_kv(WaveState<VP>& st, const bf16x8 (&qf)[KP / 32], const bf16_t* __restrict__ kpage,
+                                               const bf16_t* __restrict__ vpage, int q_pos, int key0, int valid_keys,
+                                               bool all_visible, float scale, float cap) {
+    bf16x8 kf[4][KP / 32], vf[VP / 16][2];
+    load_keys<KP>(kf, kpage);
+    load_values<VP>(vf, vpage);
+    f32x4 s[4];
+    page_scores<KP>(s, kf, qf);
+    bf16x8 pf[2];
+    float corr;
+    if (all_visible) softmax_page_bent<false, VP>(s, st, scale, cap, q_pos, key0, pf, corr);
+    else             softmax_page_bent<true, VP>(s, st, scale, cap, q_pos, key0, pf, corr);
+    weigh_values<VP>(st, vf, pf, corr, valid_keys);
+}
+
+// What finishes a row: the sink's share of the denominator (exp(0 - max), the maximum being in units of
+// log2) and the head's gate.  Returns the factor on the unnormalised output.
+__device__ __forceinline__ float finish_factor(float m, float l, int unit_sink, const float* gate_logit) {
+    if (unit_sink) l += __builtin_amdgcn_exp2f(-m);
+    float f = l > 0.f ? 1.0f / l : 0.f;
+    if (gate_logit) f *= 1.0f / (1.0f + expf(-*gate_logit));
+    return f;
+}
+
+// ---------------------------------------------------------------- prefill
+// grid (tiles of 64 tokens over all sequences, heads); wave w takes rows 16 w .. 16 w + 15 of the tile.
+template <int KS, int VB>
+__global__ __launch_bounds__(kAttnWaves * kWave) void capped_prefill_kernel(
+        bf16_t* __restrict__ out, const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_pool,
+        const bf16_t* __restrict__ v_pool, const int* __restrict__ table, int table_stride, const int* __restrict__ cu,
+        const int* __restrict__ tok_pos, int batch, int n_heads, int n_kv_heads, int group, float scale, float cap,
+        int unit_sink, const float* __restrict__ gate, int gate_stride) {
+    constexpr int KP = 32 * KS, VP = 16 * VB;
+    int tile = blockIdx.x, b = 0, first = 0;
+    for (; b < batch; ++b) {
+        const int tiles = (cu[b + 1] - cu[b] + 63) / 64;
+        if (tile < tiles) { first = cu[b] + tile * 64; break; }
+        tile -= tiles;
+    }
+    if (b >= batch) return;
+    const int h = blockIdx.y, kvh = h / group;
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int c = lane & 15, g = lane >> 4;
+    const int row0 = first + 16 * wave;
+    const int seq_end = cu[b + 1];
+    if (row0 >= seq_end) return;
+    const int rows = min(16, seq_end - row0);
+    const bool col_ok = c < rows;
+    const int my_row = row0 + (col_ok ? c : 0);
+    const int q_pos = col_ok ? tok_pos[my_row] : -1;
+    const int last_pos = tok_pos[row0 + rows - 1];
+    const int first_pos = tok_pos[row0];
+    const int written = tok_pos[seq_end - 1] + 1;
+
+    bf16x8 qf[KS];
+    const bf16_t* qrow = q + (size_t)my_row * q_stride + (size_t)h * KP + 8 * g;
+#pragma unroll
+    for (int sk = 0; sk < KS; ++sk) qf[sk] = col_ok ? ld_frag(qrow + 32 * sk) : zero_frag();
+
+    WaveState<VP> st;
+    st.init();
+    const int n_pages = last_pos / kPageTokens + 1;
+    for (int pi = 0; pi < n_pages; ++pi) {
+        const int key0 = pi * kPageTokens;
+        const size_t page = ((size_t)table[(size_t)b * table_stride + pi] * n_kv_heads + kvh) * kPageTokens;
+        attend_page_kv<KP, VP>(st, qf, k_pool + page * KP, v_pool + page * VP, q_pos, key0, min(kPageTokens, written - key0),
+                               rows == 16 && key0 + kPageTokens - 1 <= first_pos, scale, cap);
+    }
+    if (!col_ok) return;
+    const float f = finish_factor(st.m, st.l, unit_sink, gate ? gate + (size_t)my_row * gate_stride + h : nullptr);
+    bf16_t* orow = out + ((size_t)my_row * n_heads + h) * VP;
+#pragma unroll
+    for (int db = 0; db < VB; ++db) {
+        uint2 u;
+        u.x = pack_bf16(st.acc[db][0] * f, st.acc[db][1] * f);
+        u.y = pack_bf16(st.acc[db][2] * f, st.acc[db][3] * f);
+        *reinterpret_cast<uint2*>(orow + 16 * db + 4 * g) = u;
+    }
+}
+
+// ---------------------------------------------------------------- decode
+// grid (batch, kv heads, blocks along the context); wave w of a block takes pages first + w, first + w + 4, ...
+// (ppw of them).  One block along the context: the block writes the output; else partial
+// [batch][heads][grid.z][VP + 2] floats (max, sum, unnormalised output).  LDS: 4 * (group * (VP + 1) + 32) floats.
+template <int KS, int VB>
+__global__ __launch_bounds__(kAttnWaves * kWave) void capped_decode_kernel(
+        bf16_t* __restrict__ out, float* __restrict__ partial, const bf16_t* __restrict__ q, int q_stride,
+        const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool, const int* __restrict__ table, int table_stride,
+        const int* __restrict__ tok_pos, int n_heads, int n_kv_heads, int group, float scale, float cap, int ppw,
+        int unit_sink, const float* __restrict__ gate, int gate_stride) {
+    constexpr int KP = 32 * KS, VP = 16 * VB, WAVES = kAttnWaves;
+    extern __shared__ float lds[];
+    float* lds_m = lds;
+    float* lds_l = lds + WAVES * 16;
+    float* lds_o = lds + WAVES * 32;                      // [WAVES][group][VP + 1]
+    const int b = blockIdx.x, kvh = blockIdx.y, z = blockIdx.z;
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int c = lane & 15, g = lane >> 4;
+    const int pos = tok_pos[b];
+    const int n_pages = pos / kPageTokens + 1;
+    const int first_page = z * WAVES * ppw;
+    if (first_page >= n_pages) return;
+    const int* row = table + (size_t)b * table_stride;
+
+    WaveState<VP> st;
+    st.init();
+    const bool col_ok = c < group;
+    bf16x8 qf[KS];
+    const bf16_t* qrow = q + (size_t)b * q_stride + (size_t)(kvh * group + (col_ok ? c : 0)) * KP + 8 * g;
+#pragma unroll
+    for (int sk = 0; sk < KS; ++sk) qf[sk] = col_ok ? ld_frag(qrow + 32 * sk) : zero_frag();
+    for (int j = 0; j < ppw; ++j) {
+        const int pi = first_page + wave + WAVES * j;
+        if (pi >= n_pages) break;
+        const int key0 = pi * kPageTokens;
+        const size_t page = ((size_t)row[pi] * n_kv_heads + kvh) * kPageTokens;
+        attend_page_kv<KP, VP>(st, qf, k_pool + page * KP, v_pool + page * VP, col_ok ? pos : -1, key0,
+                               min(kPageTokens, pos - key0 + 1), key0 + kPageTokens - 1 <= pos, scale, cap);
+    }
+    if (g == 0) { lds_m[wave * 16 + c] = st.m; lds_l[wave * 16 + c] = st.l; }
+    if (col_ok) {
+        float* dst = lds_o + ((size_t)wave * group + c) * (VP + 1);
+#pragma unroll
+        for (int db = 0; db < VB; ++db)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) dst[16 * db + 4 * g + r] = st.acc[db][r];
+    }
+    __syncthreads();
+    const int n_z = gridDim.z;
+    for (int idx = threadIdx.x; idx < group * VP; idx += blockDim.x) {
+        const int col = idx / VP, d = idx % VP;
+        float m = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) m = fmaxf(m, lds_m[w * 16 + col]);
+        float l = 0.f, o = 0.f;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) {
+            const float mw = lds_m[w * 16 + col];
+            const float f = (mw == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mw - m);
+            l += lds_l[w * 16 + col] * f;
+            o += lds_o[((size_t)w * group + col) * (VP + 1) + d] * f;
+        }
+        const int head = kvh * group + col;
+        if (n_z == 1) {
+            const float f = finish_factor(m, l, unit_sink, gate ? gate + (size_t)b * gate_stride + head : nullptr);
+            out[((size_t)b * n_heads + head) * VP + d] = f32_to_bf16(o * f);
+        } else {
+            float* dst = partial + (((size_t)b * n_heads + head) * n_z + z) * (VP + 2);
+            dst[2 + d] = o;
+            if (d == 0) { dst[0] = m; dst[1] = l; }
+        }
+    }
+}
+
+// grid (batch, heads), VP threads: thread d adds dimension d of the blocks' partial results in ascending order.
+template <int VB>
+__global__ __launch_bounds__(16 * VB) void capped_merge_kernel(bf16_t* __restrict__ out, const float* __restrict__ partial,
+                                                               const int* __restrict__ tok_pos, int n_heads, int n_z,
+                                                               int pages_per_block, int unit_sink,
+                                                               const float* __restrict__ gate, int gate_stride) {
+    constexpr int VP = 16 * VB;
+    const int b = blockIdx.x, h = blockIdx.y, d = threadIdx.x;
+    const int n_pages = tok_pos[b] / kPageTokens + 1;
+    const int used = min(n_z, (n_pages + pages_per_block - 1) / pages_per_block);
+    const float* src = partial + ((size_t)b * n_heads + h) * n_z * (VP + 2);
+    float m = -INFINITY;
+    for (int z = 0; z < used; ++z) m = fmaxf(m, src[(size_t)z * (VP + 2)]);
+    float l = 0.f, o = 0.f;
+    for (int z = 0; z < used; ++z) {
+        const float* p = src + (size_t)z * (VP + 2);
+        const float f = (p[0] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(p[0] - m);
+        l += p[1] * f;
+        o += p[2 + d] * f;
+    }
+    const float f = finish_factor(m, l, unit_sink, gate ? gate + (size_t)b * gate_stride + h : nullptr);
+    out[((size_t)b * n_heads + h) * VP + d] = f32_to_bf16(o * f);
+}
+
+// ---------------------------------------------------------------- entry points
+static int capped_units() {
+    static int units = 0;
+    if (units == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) units = prop.multiProcessorCount;
+        if (units <= 0) units = 256;
+    }
+    return units;
+}
+
+static bool capped_shape_ok(int n_heads, int n_kv_heads, int dk, int dv) {
+    if (n_heads <= 0 || n_kv_heads <= 0 || n_heads % n_kv_heads || n_heads / n_kv_heads > 16) return false;
+    const bool k_ok = dk == 64 || dk == 96 || dk == 128;
+    const bool v_ok = dv == 64 || dv == 80 || dv == 96 || dv == 128;
+    return k_ok && v_ok;
+}
+
+// pages a wave takes in a decode step: as few as leave no more than two blocks a compute unit
+static int capped_pages_per_wave(int batch, int n_kv_heads, int table_width) {
+    const int room = 2 * capped_units();
+    for (int ppw = 1; ppw < 16; ++ppw) {
+        const int n_z = (table_width + kAttnWaves * ppw - 1) / (kAttnWaves * ppw);
+        if ((long long)batch * n_kv_heads * n_z <= room) return ppw;
+    }
+    return 16;
+}
+
+#define CAPPED_SHAPES(DO) \
+    if (dk == 64 && dv == 64) DO(2, 4); else if (dk == 64 && dv == 80) DO(2, 5); else if (dk == 64 && dv == 96) DO(2, 6); \
+    else if (dk == 64 && dv == 128) DO(2, 8); else if (dk == 96 && dv == 64) DO(3, 4); else if (dk == 96 && dv == 80) DO(3, 5); \
+    else if (dk == 96 && dv == 96) DO(3, 6); else if (dk == 96 && dv == 128) DO(3, 8); else if (dk == 128 && dv == 64) DO(4, 4); \
+    else if (dk == 128 && dv == 80) DO(4, 5); else if (dk == 128 && dv == 96) DO(4, 6); else DO(4, 8);
+
+// -2: a shape these kernels do not take (the caller uses the kernel for any shape)
+LLOGOS_EXPORT int llogos_capped_attn_prefill_bf16(void* out, const void* q, int q_stride, const void* k_pool, const void* v_pool,
+                                                  const int* table, int table_stride, const int* cu, const int* tok_pos,
+                                                  int batch, int n_tiles, int n_heads, int n_kv_heads, int dk, int dv, float scale,
+                                                  float softcap, int unit_sink, const float* gate, int gate_stride,
+                                                  hipStream_t stream) {
+    if (batch <= 0 || n_tiles <= 0 || softcap < 0.f || (gate && gate_stride < n_heads)) return LLOGOS_BAD_ARGUMENT;
+    if (!capped_shape_ok(n_heads, n_kv_heads, dk, dv) || q_stride % 8) return LLOGOS_UNSUPPORTED;
+    dim3 grid(n_tiles, n_heads);
+    const int group = n_heads / n_kv_heads;
+#define PRE(KS, VB) capped_prefill_kernel<KS, VB><<<grid, kAttnWaves * kWave, 0, stream>>>((bf16_t*)out, (const bf16_t*)q, q_stride, \
+        (const bf16_t*)k_pool, (const bf16_t*)v_pool, table, table_stride, cu, tok_pos, batch, n_heads, n_kv_heads, group, scale, \
+        softcap, unit_sink, gate, gate_stride)
+    CAPPED_SHAPES(PRE)
+#undef PRE
+    return LLOGOS_LAUNCH_CHECK();
+}
+
+LLOGOS_EXPORT long long llogos_capped_attn_decode_workspace(int batch, int n_heads, int n_kv_heads, int dv, int table_width) {
+    if (batch <= 0 || n_heads <= 0 || n_kv_heads <= 0 || dv <= 0 || table_width <= 0) return 0;
+    const int ppw = capped_pages_per_wave(batch, n_kv_heads, table_width);
+    const int n_z = (table_width + kAttnWaves * ppw - 1) / (kAttnWaves * ppw);
+    return n_z > 1 ? (long long)batch * n_heads * n_z * (dv + 2) : 0;
+}
+
+LLOGOS_EXPORT int llogos_capped_attn_decode_bf16(void* out, const void* q, int q_stride, const void* k_pool, const void* v_pool,
+                                                 const int* table, int table_stride, int table_width, const int* tok_pos,
+                                                 int batch, int n_heads, int n_kv_heads, int dk, int dv, float scale,
+                                                 float softcap, int unit_sink, const float* gate, int gate_stride,
+                                                 float* workspace, long long workspace_floats, hipStream_t stream) {
+    if (batch <= 0 || table_width <= 0 || softcap < 0.f || (gate && gate_stride < n_heads)) return LLOGOS_BAD_ARGUMENT;
+    if (!capped_shape_ok(n_heads, n_kv_heads, dk, dv) || q_stride % 8) return LLOGOS_UNSUPPORTED;
+    const int group = n_heads / n_kv_heads;
+    const int ppw = capped_pages_per_wave(batch, n_kv_heads, table_width);
+    const int n_z = (table_width + kAttnWaves * ppw - 1) / (kAttnWaves * ppw);
+    if (n_z > 1 && (!workspace || workspace_floats < (long long)batch * n_heads * n_z * (dv + 2))) return LLOGOS_TOO_LARGE;
+    dim3 grid(batch, n_kv_heads, n_z);
+    const size_t lds = (size_t)kAttnWaves * (group * (dv + 1) + 32) * sizeof(float);
+#define DEC(KS, VB) capped_decode_kernel<KS, VB><<<grid, kAttnWaves * kWave, lds, stream>>>((bf16_t*)out, workspace, (const bf16_t*)q, \
+        q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, table, table_stride, tok_pos, n_heads, n_kv_heads, group, scale, \
+        softcap, ppw, unit_sink, gate, gate_stride)
+    CAPPED_SHAPES(DEC)
+#undef DEC
+    if (n_z > 1) {
+        dim3 mgrid(batch, n_heads);
+#define MRG(VB) capped_merge_kernel<VB><<<mgrid, 16 * VB, 0, stream>>>((bf16_t*)out, workspace, tok_pos, n_heads, n_z, kAttnWaves * ppw, \
+        unit_sink, gate, gate_stride)
+        if (dv == 64) MRG(4); else if (dv == 80) MRG(5); else if (dv == 96) MRG(6); else MRG(8);
+#undef MRG
+    }
+    return LLOGOS_LAUNCH_CHECK();
+}

@@ -1602,6 +1602,52 @@ def attention(ctx, q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool:
                              n_heads, n_kv_heads, head_dim, scale, window, sinks)
 
 
+def capped_attention(ctx, q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, table: torch.Tensor, n_heads: int,
+                     n_kv_heads: int, head_dim: int, v_dim: int, scale: float, softcap: float = 0.0,
+                     unit_sink: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Causal attention of the step's query rows q [T, n_heads * head_dim] over their sequences' pages, for keys of
+    head_dim and values of v_dim dimensions: scores bent to softcap * tanh(score / softcap) (softcap > 0), a sink of
+    score 0 in the softmax's denominator (unit_sink: float32 zeros [n_heads]), head h's output times
+    sigmoid(gate[t, h]) (gate float32 [T, >= n_heads], maybe a view of wider rows).  Returns [T, n_heads * v_dim].
+    bfloat16 with head sizes the matrix-core kernels take runs there; everything else in the kernel for any shape."""
+    T = ctx.n_tokens
+    if q.dtype == torch.bfloat16 and q.dim() == 2 and q.is_contiguous():
+        kd, vd = _page_dims(k_pool, v_pool, n_kv_heads, "attention")
+        if kd == head_dim and vd == v_dim and v_pool is not None:
+            _dev(table, ctx.tok_pos)
+            _i32(table, "table")
+            _need(tuple(q.shape) == (T, n_heads * head_dim), "attention: q must be [T, heads * head_dim]")
+            gate_stride = 0
+            if gate is not None:
+                _need(gate.is_cuda and gate.dtype == torch.float32 and gate.dim() == 2 and gate.shape[0] == T
+                      and gate.shape[1] >= n_heads and gate.stride(1) == 1, "attention: gate must be float32 [T, n_heads]")
+                gate_stride = gate.stride(0) if T > 1 else max(n_heads, gate.stride(0))
+            out = torch.empty((T, n_heads * v_dim), dtype=torch.bfloat16, device=q.device)
+            lib = _lib()
+            sink = 1 if unit_sink is not None else 0
+            if ctx.is_decode:
+                width = table.shape[1]
+                _need(table.shape[0] == T and ctx.tok_pos.numel() == T, "attention: one table row and position a sequence")
+                ws = _attn_workspace(q.device, lib.llogos_capped_attn_decode_workspace(T, n_heads, n_kv_heads, v_dim, width))
+                code = lib.llogos_capped_attn_decode_bf16(
+                    _p(out), _p(q), q.stride(0), _p(k_pool), _p(v_pool), _p(table), table.stride(0), width, _p(ctx.tok_pos), T,
+                    n_heads, n_kv_heads, head_dim, v_dim, ctypes.c_float(scale), ctypes.c_float(softcap), sink, _p(gate),
+                    gate_stride, _p(ws), ctypes.c_longlong(ws.numel()), _stream())
+            else:
+                cu = ctx.cu_dev
+                _need(cu is not None and cu.numel() == ctx.batch + 1, "attention: the step's token offsets are missing")
+                n_tiles = sum(-(-(ctx.cu_seqlens[i + 1] - ctx.cu_seqlens[i]) // 64) for i in range(ctx.batch))
+                code = lib.llogos_capped_attn_prefill_bf16(
+                    _p(out), _p(q), q.stride(0), _p(k_pool), _p(v_pool), _p(table), table.stride(0), _p(cu), _p(ctx.tok_pos),
+                    ctx.batch, n_tiles, n_heads, n_kv_heads, head_dim, v_dim, ctypes.c_float(scale), ctypes.c_float(softcap),
+                    sink, _p(gate), gate_stride, _stream())
+            if code != -2:
+                _check(code, "capped_attention")
+                return out
+    return attention_generic(q, n_heads * head_dim, k_pool, v_pool, table, ctx.tok_seq, ctx.tok_pos, n_heads, n_kv_heads,
+                             head_dim, scale, v_dim=v_dim, head_sink=unit_sink, softcap=softcap, gate=gate)
+
+
 # ----------------------------------------------------------------------------
 # sampling
 # ----------------------------------------------------------------------------

@@ -114,9 +114,8 @@ class CappedAttention(Mixer):
                           self.q_norm_w, self.k_norm_w, self.eps, self.temp_coef, self.temp_every, cache.k_pool, cache.v_pool,
                           cache.table, writes=cache.writes)
         mark(ctx, "prepare")
-        a = K.attention_generic(q, nq, cache.k_pool, cache.v_pool, cache.table, ctx.tok_seq, ctx.tok_pos, self.n_heads,
-                                self.n_kv_heads, self.head_dim, self.scale, v_dim=self.v_dim, head_sink=self.sink,
-                                softcap=self.softcap, gate=gate)
+        a = K.capped_attention(ctx, q, cache.k_pool, cache.v_pool, cache.table, self.n_heads, self.n_kv_heads, self.head_dim,
+                               self.v_dim, self.scale, self.softcap, self.sink, gate)
         mark(ctx, "attention")
         out = self.o.add_to(a, residual) if residual is not None else None
         if out is None:
