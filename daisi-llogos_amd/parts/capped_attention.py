@@ -92,6 +92,8 @@ class CappedAttention(Mixer):
             self.q_norm_w, self.k_norm_w = f32("q.norm"), f32("k.norm")
         if self.conv_taps:
             self.conv_w = torch.cat([f32("q.conv"), f32("k.conv"), f32("v.conv")], dim=0).contiguous()     # [W, taps]
+            # one tap reads no row before the present one: the kernel is handed a state without rows
+            self._no_state = torch.zeros((1, 0, self.W), dtype=torch.float32, device=rt.device)
         if self.unit_sink:
             self.sink = torch.zeros(self.n_heads, dtype=torch.float32, device=rt.device)     # a sink whose score is 0
 
@@ -108,7 +110,8 @@ class CappedAttention(Mixer):
             # (a run that reads another's cache has no state of its own to convolve with: not built)
             if cache.state is None and self.conv_taps > 1:
                 raise RuntimeError("a convolution behind the projections needs the run's own state")
-            rows = K.causal_conv(ctx, rows[:, :W], self.conv_w, cache.state, torch.float32, add_input=False)
+            state = cache.state if self.conv_taps > 1 else self._no_state
+            rows = K.causal_conv(ctx, rows[:, :W], self.conv_w, state, torch.float32, add_input=False)
             mark(ctx, "conv")
         q = K.qkv_prepare(ctx, rows, self.qkv.bias, self.rt.dtype, self.n_heads, self.n_kv_heads, self.head_dim, self.v_dim,
                           self.q_norm_w, self.k_norm_w, self.eps, self.temp_coef, self.temp_every, cache.k_pool, cache.v_pool,

@@ -216,3 +216,13 @@ def load_folder(path: str):
     for k, t in load_file(os.path.join(path, "model.safetensors")).items():
         w[k] = t.numpy() if t.dtype in (torch.int32, torch.int64) else t.to(torch.float64).numpy()
     return cfg, w
+
+
+def generate_greedy(cfg: dict, w: dict, prompt, n: int) -> list:
+    """n tokens, each the first largest logit after everything before it (the whole sequence is run again each time)."""
+    seq, out = list(prompt), []
+    for _ in range(n):
+        tok = int(np.argmax(forward(cfg, w, seq)[-1]))
+        out.append(tok)
+        seq.append(tok)
+    return out

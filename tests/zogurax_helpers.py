@@ -1,0 +1,73 @@
+"""Shared by the Zogurax tests: model folders of the small configurations (random weights, with the
+query and key matrices scaled up so that attention is sharp and a lost or extra key, a lost sink or
+a wrong position shows), the plain implementation's logits, and the bounds."""
+import functools
+import importlib
+import os
+import tempfile
+
+import numpy as np
+
+import plain_zogurax as pz
+import zogurax_configs as zc
+
+llogos = importlib.import_module("daisi-llogos_amd")
+_tmp = tempfile.TemporaryDirectory(prefix="llogos_test_zogurax_")
+SHARP = 3.0
+DTYPES = ["float32", "bfloat16"]
+# float32: the engine against float64 arithmetic, relative to the largest logit.  bfloat16: rounding of the
+# matrix products' inputs; the bound is loose, and what must not happen (a key too few, a lost state) is
+# asserted in float32 and, with a margin, on sharpened models.
+TOL = {"float32": 2e-4, "bfloat16": 0.12}
+
+
+@functools.lru_cache(maxsize=None)
+def folder(name: str, seed: int = 5) -> str:
+    from safetensors.torch import load_file, save_file
+    path = os.path.join(_tmp.name, f"{name}_{seed}")
+    llogos.write_random_model(path, zc.ALL[name], seed=seed, std=0.08)
+    file = os.path.join(path, "model.safetensors")
+    tensors = load_file(file)
+    for k in tensors:
+        if k.endswith((".mix.q", ".mix.k")):
+            tensors[k] = (tensors[k].float() * SHARP).to(tensors[k].dtype)
+        if k.endswith((".mix.q.norm", ".mix.k.norm")):
+            tensors[k] = (tensors[k].float() * 2.0).to(tensors[k].dtype)
+        if k == "loop.in":                                     # (keeps the stream's size through the passes)
+            tensors[k] = (tensors[k].float() * 6.0).to(tensors[k].dtype)
+    save_file(tensors, file)
+    return path
+
+
+@functools.lru_cache(maxsize=None)
+def plain(name: str, seed: int = 5):
+    return pz.load_folder(folder(name, seed))
+
+
+@functools.lru_cache(maxsize=None)
+def plain_logits(name: str, tokens: tuple, seed: int = 5) -> np.ndarray:
+    cfg, w = plain(name, seed)
+    return pz.forward(cfg, w, list(tokens))
+
+
+def tokens(name: str, n: int, seed: int) -> tuple:
+    rng = np.random.default_rng(seed)
+    return tuple(int(t) for t in rng.integers(0, zc.ALL[name]["vocab"], size=n))
+
+
+def engine(name: str, dtype: str, max_tokens: int = 1024, n_slots: int = 4, seed: int = 5, **options):
+    return llogos.Engine.from_folder(folder(name, seed), dtype=dtype, max_tokens=max_tokens, n_slots=n_slots, **options)
+
+
+def distance(got, want) -> float:
+    """Largest difference of the logits, relative to the largest logit's size."""
+    got, want = np.asarray(got, dtype=np.float64), np.asarray(want, dtype=np.float64)
+    assert got.shape == want.shape, f"shape {got.shape} vs {want.shape}"
+    assert np.isfinite(got).all(), "not finite"
+    return float(np.abs(got - want).max() / max(1e-9, np.abs(want).max()))
+
+
+def close(got, want, dtype: str, what: str = "") -> float:
+    d = distance(got, want)
+    assert d <= TOL[dtype], f"{what}: relative error {d:.3e} > {TOL[dtype]:.1e} ({dtype})"
+    return d
