@@ -159,16 +159,44 @@ def nipulorn_config(width, layers, vocab, ff):
             "torch_dtype": "bfloat16"}
 
 
+def zogurax_config(width, runs, vocab, ff):
+    """Layers of real sizes: the two attention forms in turn, heads of 128 dimensions (keys and values), four query
+    heads a key/value head; 16 experts of which a token takes 2, each and the shared one a third as wide as the dense
+    decoder's feed-forward (two matrices an expert instead of three, three experts a token: the same weight a token);
+    the second and third layer are gone through twice, which makes `runs` runs of `runs - 2` layers."""
+    heads = width // 128
+    moe = {"kind": "moe", "router": {"experts": 16, "top": 2}, "expert": {"ff": ff // 2}, "shared": {"ff": ff // 2}}
+    mixer = {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "softcap": 50.0,
+             "q_temp": {"coef": 0.3, "every": 128}}
+    first = {"type": "attention", "mixer": dict(mixer, conv=4), "mlp": moe}
+    second = {"type": "attention_2", "mixer": mixer, "mlp": moe}
+    return {"architecture": "Zogurax", "vocab": vocab, "width": width, "norm": {"eps": 1e-5},
+            "layers": [second if i % 2 == 0 else first for i in range(runs - 2)], "loop": {"start": 1, "stop": 3, "times": 2},
+            "torch_dtype": "bfloat16"}
+
+
+def moe_bytes_read(model, rows: int) -> int:
+    """Bytes of weights that a step of `rows` tokens reads at most: as step_weight_bytes, but of a layer's experts
+    only as many as the rows can choose."""
+    total = model.step_weight_bytes()
+    for e in model.schedule:
+        for f in model.layers[e.layer].feed_forwards():
+            if hasattr(f, "n_experts"):
+                experts = (f.up.numel() + f.down.numel()) * f.up.element_size()
+                total -= experts - experts * min(f.n_experts, rows * f.top) // f.n_experts
+    return total
+
+
 def compare_designs(args) -> int:
-    """Prefill and decode throughput of Nipulorn models of real layer sizes (random weights) and of the dense
-    decoder with the same width, depth and about the same weight bytes, and where a step's time goes part by
-    part in both.  One JSON line at the end."""
+    """Prefill and decode throughput of models of the chosen design at real layer sizes (random weights) and of the
+    dense decoder with the same width, as many layer runs and about the same weight bytes a token, and where a
+    step's time goes part by part in both.  One JSON line at the end."""
     import numpy as np
     import torch
     llogos = importlib.import_module("daisi-llogos_amd")
     rng = np.random.default_rng(0)
     sizes = [("2048 wide", 2048, 8192, 8), ("4096 wide", 4096, 14336, 8)]
-    record = {"metric": "design_comparison", "design": "Nipulorn", "against": "dense decoder (Llama sizes)", "dtype": "bf16",
+    record = {"metric": "design_comparison", "design": args.design.capitalize(), "against": "dense decoder (Llama sizes)", "dtype": "bf16",
               "data": "synthetic", "sizes": []}
 
     def measure(label, cfg, vocab):
@@ -211,7 +239,7 @@ def compare_designs(args) -> int:
             dt = timed(lambda: [step() for _ in range(args.steps)], repeat=2) / args.steps
             out[f"decode_b{batch}_tok_s"] = round(batch / dt)
             out[f"decode_b{batch}_us"] = round(dt * 1e6, 1)
-            out[f"decode_b{batch}_roofline"] = round(model.step_weight_bytes() / HBM_PEAK / dt, 3)
+            out[f"decode_b{batch}_roofline"] = round(moe_bytes_read(model, batch) / HBM_PEAK / dt, 3)
             if batch == 8:
                 probe = llogos.StepProbe()
                 probe.hold()
@@ -229,9 +257,12 @@ def compare_designs(args) -> int:
     for name, width, ff, layers in sizes:
         dense = dict(LLAMA31_8B, hidden_size=width, intermediate_size=ff, num_hidden_layers=layers, vocab_size=vocab,
                      num_attention_heads=width // 128, num_key_value_heads=max(1, width // 512), tie_word_embeddings=True)
-        # two matrices a feed-forward instead of three: half as wide again for the same weight
-        nip = nipulorn_config(width, layers, vocab, ff * 3 // 2)
-        record["sizes"].append({"size": name, "layers": layers, "nipulorn": measure(f"nipulorn {name}", nip, vocab),
+        if args.design == "zogurax":
+            other = zogurax_config(width, layers, vocab, ff)
+        else:
+            # two matrices a feed-forward instead of three: half as wide again for the same weight
+            other = nipulorn_config(width, layers, vocab, ff * 3 // 2)
+        record["sizes"].append({"size": name, "layers": layers, args.design: measure(f"{args.design} {name}", other, vocab),
                                 "dense": measure(f"dense {name}", dense, vocab)})
     print(json.dumps(record), flush=True)
     return 0
@@ -239,7 +270,7 @@ def compare_designs(args) -> int:
 
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser()
-    ap.add_argument("--design", choices=["nipulorn"], default=None,
+    ap.add_argument("--design", choices=["nipulorn", "zogurax"], default=None,
                     help="instead of the default run: this design beside the dense decoder at equal sizes (prefill, decode, parts)")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=248)   # + 8 warm-up = 256 new tokens

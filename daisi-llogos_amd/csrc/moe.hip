@@ -195,3 +195,211 @@ LLOGOS_EXPORT int llogos_moe_combine(float* out, const float* y, const int* wher
                                                      gate_parts, (size_t)gate_part_stride, T, W);
     return LLOGOS_LAUNCH_CHECK();
 }
+
+// ---------------------------------------------------------------- bfloat16 on the matrix cores
+// The same product with v_mfma_f32_16x16x32_bf16: the first operand holds 16 rows of the expert's matrix, the
+// second 16 sorted rows of activations, so that a lane ends with four neighbouring outputs of one row:
+// D[n = 4 g + r][m = c] for lane (c = lane & 15, g = lane >> 4).  A lane's share of an operand is 8 values of k,
+// 16 bytes.  Two forms:
+//   few rows  tiles of 16 sorted rows; a block of four waves owns 16 rows of the matrix, its waves take the
+//             steps of 32 k in turn (together whole cache lines), straight from memory into operands, and LDS
+//             adds the four waves' sums in order;
+//   tiles     64 or 128 sorted rows x 128 rows of the matrix, stages of 64 k through LDS (rows 160 bytes
+//             apart: fragment reads without bank conflicts), the next stage's loads in registers meanwhile.
+// Sums depend on k's order alone, as above.  K must be a multiple of 8 and N of 4.
+typedef __bf16 moe_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float moe_f32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ moe_bf16x8 moe_frag(const bf16_t* p) {
+    return __builtin_bit_cast(moe_bf16x8, *reinterpret_cast<const uint4*>(p));
+}
+__device__ __forceinline__ moe_bf16x8 moe_zero() { return __builtin_bit_cast(moe_bf16x8, make_uint4(0, 0, 0, 0)); }
+
+__device__ __forceinline__ void moe_store4(float* p, float a, float b, float c, float d) {
+    *reinterpret_cast<float4*>(p) = make_float4(a, b, c, d);
+}
+__device__ __forceinline__ void moe_store4(bf16_t* p, float a, float b, float c, float d) {
+    uint2 u;
+    u.x = (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16);
+    u.y = (uint32_t)f32_to_bf16(c) | ((uint32_t)f32_to_bf16(d) << 16);
+    *reinterpret_cast<uint2*>(p) = u;
+}
+
+// which tile of `rows` sorted rows is this block's: expert, first row, end of the expert's segment (expert -1: none)
+__device__ __forceinline__ void moe_find_tile(const int* __restrict__ seg, int E, int rows, int tile, int& expert, int& first, int& end) {
+    expert = -1; first = 0; end = 0;
+    for (int e = 0; e < E; ++e) {
+        const int lo = seg[e], hi = seg[e + 1];
+        const int tiles = (hi - lo + rows - 1) / rows;
+        if (tile < tiles) { expert = e; first = lo + tile * rows; end = hi; return; }
+        tile -= tiles;
+    }
+}
+
+template <typename TO>
+__global__ __launch_bounds__(256) void moe_few_kernel(TO* __restrict__ out, const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
+                                                      const int* __restrict__ order, const int* __restrict__ seg, int E, int top,
+                                                      int gather, int N, int K, int lda, int act, float scale) {
+    __shared__ float red[3][kWave][4];
+    __shared__ int s_tile[3];
+    if (threadIdx.x == 0) moe_find_tile(seg, E, 16, blockIdx.y, s_tile[0], s_tile[1], s_tile[2]);
+    __syncthreads();
+    const int e = s_tile[0], m0 = s_tile[1], m_end = s_tile[2];
+    if (e < 0) return;
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int c = lane & 15, g = lane >> 4;
+    const int n0 = blockIdx.x * 16;
+    const int m = m0 + c;
+    const bf16_t* arow = m < m_end ? a + (size_t)(gather ? order[m] / top : m) * lda + 8 * g : nullptr;
+    const bf16_t* wrow = n0 + c < N ? w + ((size_t)e * N + n0 + c) * K + 8 * g : nullptr;
+    moe_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    const int steps = (K + 31) / 32;
+#pragma unroll 4
+    for (int s = wave; s < steps; s += 4) {
+        const int k = 32 * s;
+        const bool in = k + 8 * g < K;
+        const moe_bf16x8 wf = (wrow && in) ? moe_frag(wrow + k) : moe_zero();
+        const moe_bf16x8 af = (arow && in) ? moe_frag(arow + k) : moe_zero();
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, af, acc, 0, 0, 0);
+    }
+    if (wave > 0) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) red[wave - 1][lane][r] = acc[r];
+    }
+    __syncthreads();
+    if (wave > 0) return;
+    float v[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        v[r] = ((acc[r] + red[0][lane][r]) + red[1][lane][r]) + red[2][lane][r];
+        if (act == 1) { v[r] = fmaxf(v[r], 0.f); v[r] *= v[r]; }
+        v[r] *= scale;
+    }
+    const int n = n0 + 4 * g;
+    if (m < m_end && n < N) moe_store4(out + (size_t)m * N + n, v[0], v[1], v[2], v[3]);
+}
+
+constexpr int kMoeBN = 128, kMoeBK = 64, kMoeLd = 80;      // LDS rows of 64 values, 160 bytes apart
+
+template <int BM, typename TO>
+__global__ __launch_bounds__(256) void moe_tiles_kernel(TO* __restrict__ out, const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
+                                                        const int* __restrict__ order, const int* __restrict__ seg, int E, int top,
+                                                        int gather, int N, int K, int lda, int act, float scale) {
+    constexpr int CA = BM * 8 / 256, CW = kMoeBN * 8 / 256;           // 16-byte pieces a thread copies a stage
+    constexpr int WN = BM == 128 ? 64 : 32, NT = WN / 16, MT = 4;     // a wave's part: 64 rows x WN columns of the tile
+    __shared__ __attribute__((aligned(16))) bf16_t As[BM * kMoeLd];
+    __shared__ __attribute__((aligned(16))) bf16_t Ws[kMoeBN * kMoeLd];
+    __shared__ int src_row[BM];
+    __shared__ int s_tile[3];
+    const int tid = threadIdx.x;
+    if (tid == 0) moe_find_tile(seg, E, BM, blockIdx.y, s_tile[0], s_tile[1], s_tile[2]);
+    __syncthreads();
+    const int e = s_tile[0], m0 = s_tile[1], m_end = s_tile[2];
+    if (e < 0) return;
+    if (tid < BM) {
+        const int r = m0 + tid;
+        src_row[tid] = r < m_end ? (gather ? order[r] / top : r) : -1;
+    }
+    __syncthreads();
+    const int lane = tid & (kWave - 1), wave = tid / kWave;
+    const int c = lane & 15, g = lane >> 4;
+    const int wm = BM == 128 ? wave >> 1 : 0, wn = BM == 128 ? wave & 1 : wave;
+    const int n0 = blockIdx.x * kMoeBN;
+    const bf16_t* we = w + (size_t)e * N * K;
+
+    const bf16_t* pa[CA];
+    const bf16_t* pw[CW];
+    int ka[CA], kw[CW];
+#pragma unroll
+    for (int j = 0; j < CA; ++j) {
+        const int q = tid + 256 * j, row = q >> 3;
+        ka[j] = (q & 7) * 8;
+        pa[j] = src_row[row] >= 0 ? a + (size_t)src_row[row] * lda + ka[j] : nullptr;
+    }
+#pragma unroll
+    for (int j = 0; j < CW; ++j) {
+        const int q = tid + 256 * j, row = q >> 3;
+        kw[j] = (q & 7) * 8;
+        pw[j] = n0 + row < N ? we + (size_t)(n0 + row) * K + kw[j] : nullptr;
+    }
+    uint4 ra[CA], rw[CW];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int j = 0; j < CA; ++j)
+            ra[j] = (pa[j] && k0 + ka[j] < K) ? *reinterpret_cast<const uint4*>(pa[j] + k0) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+        for (int j = 0; j < CW; ++j)
+            rw[j] = (pw[j] && k0 + kw[j] < K) ? *reinterpret_cast<const uint4*>(pw[j] + k0) : make_uint4(0, 0, 0, 0);
+    };
+    moe_f32x4 acc[NT][MT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = moe_f32x4{0.f, 0.f, 0.f, 0.f};
+
+    fetch(0);
+    for (int k0 = 0; k0 < K; k0 += kMoeBK) {
+#pragma unroll
+        for (int j = 0; j < CA; ++j) {
+            const int q = tid + 256 * j;
+            *reinterpret_cast<uint4*>(As + (q >> 3) * kMoeLd + (q & 7) * 8) = ra[j];
+        }
+#pragma unroll
+        for (int j = 0; j < CW; ++j) {
+            const int q = tid + 256 * j;
+            *reinterpret_cast<uint4*>(Ws + (q >> 3) * kMoeLd + (q & 7) * 8) = rw[j];
+        }
+        __syncthreads();
+        if (k0 + kMoeBK < K) fetch(k0 + kMoeBK);
+#pragma unroll
+        for (int ks = 0; ks < kMoeBK / 32; ++ks) {
+            moe_bf16x8 af[MT], wf[NT];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) af[mt] = moe_frag(As + (wm * 64 + mt * 16 + c) * kMoeLd + ks * 32 + 8 * g);
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) wf[nt] = moe_frag(Ws + (wn * WN + nt * 16 + c) * kMoeLd + ks * 32 + 8 * g);
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+                    acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[nt], af[mt], acc[nt][mt], 0, 0, 0);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int m = m0 + wm * 64 + mt * 16 + c;
+        if (m >= m_end) continue;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            const int n = n0 + wn * WN + nt * 16 + 4 * g;
+            if (n >= N) continue;
+            float v[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                v[r] = acc[nt][mt][r];
+                if (act == 1) { v[r] = fmaxf(v[r], 0.f); v[r] *= v[r]; }
+                v[r] *= scale;
+            }
+            moe_store4(out + (size_t)m * N + n, v[0], v[1], v[2], v[3]);
+        }
+    }
+}
+
+// form 0: few rows (tiles of 16); 1: tiles of 64 rows; 2: tiles of 128 rows.  -2 for shapes these do not take.
+LLOGOS_EXPORT int llogos_moe_product_bf16(void* out, int out_dtype, const void* a, const void* w, const int* order, const int* seg,
+                                          int E, int top, int gather, int P, int N, int K, int lda, int act, float scale, int form,
+                                          hipStream_t stream) {
+    if (P <= 0 || N <= 0 || K <= 0 || E <= 0 || top <= 0 || lda < K || act < 0 || act > 1 || form < 0 || form > 2) return LLOGOS_BAD_ARGUMENT;
+    if ((K % 8) || (N % 4) || (lda % 8) || ((uintptr_t)a % 16) || ((uintptr_t)w % 16) || ((uintptr_t)out % 16)) return LLOGOS_UNSUPPORTED;
+    if (out_dtype != DT_F32 && out_dtype != DT_BF16) return LLOGOS_BAD_ARGUMENT;
+    const int rows = form == 0 ? 16 : (form == 1 ? 64 : 128);
+    const int row_tiles = (P + rows - 1) / rows + E;
+#define MOE_GO(KERNEL, NB, TO) KERNEL<<<dim3((N + NB - 1) / NB, row_tiles), 256, 0, stream>>>((TO*)out, (const bf16_t*)a, (const bf16_t*)w, \
+        order, seg, E, top, gather, N, K, lda, act, scale)
+    if (form == 0) { if (out_dtype == DT_F32) MOE_GO(moe_few_kernel<float>, 16, float); else MOE_GO(moe_few_kernel<bf16_t>, 16, bf16_t); }
+    else if (form == 1) { if (out_dtype == DT_F32) MOE_GO((moe_tiles_kernel<64, float>), kMoeBN, float); else MOE_GO((moe_tiles_kernel<64, bf16_t>), kMoeBN, bf16_t); }
+    else { if (out_dtype == DT_F32) MOE_GO((moe_tiles_kernel<128, float>), kMoeBN, float); else MOE_GO((moe_tiles_kernel<128, bf16_t>), kMoeBN, bf16_t); }
+#undef MOE_GO
+    return LLOGOS_LAUNCH_CHECK();
+}

@@ -595,6 +595,8 @@ def activation(x: torch.Tensor, kind: str, out_dtype: torch.dtype, a: float = 0.
 # experts chosen by a table over token ids
 # ----------------------------------------------------------------------------
 MOE_MAX_EXPERTS = 1024
+MOE_FEW_PAIRS = 256          # up to so many (token, choice) pairs a step the experts' product streams the matrices in tiles of 16 rows
+MOE_PRODUCT = "auto"         # "auto": chosen by the step; "plain", "few", "tiles64", "tiles128" force a form (tests)
 
 
 def moe_route(ids: torch.Tensor, table: torch.Tensor, n_experts: int):
@@ -625,6 +627,17 @@ def moe_product(a: torch.Tensor, w: torch.Tensor, order: torch.Tensor, seg: torc
     _need(gather or a.shape[0] == P, "moe_product: sorted rows must be as many as pairs")
     _need(not gather or a.shape[0] * top == P, "moe_product: token rows times choices must be the pairs")
     out = torch.empty((P, N), dtype=out_dtype, device=a.device)
+    if a.dtype == torch.bfloat16 and MOE_PRODUCT != "plain" and a.stride(1) == 1:
+        # on the matrix cores: tiles of 16 sorted rows straight from memory for steps of few rows, tiles of 64 or
+        # 128 rows through LDS where an expert's segment is long enough on average to fill them
+        form = 0 if P <= MOE_FEW_PAIRS else (2 if P >= 96 * E else 1)
+        if MOE_PRODUCT in ("few", "tiles64", "tiles128"):
+            form = ("few", "tiles64", "tiles128").index(MOE_PRODUCT)
+        code = _lib().llogos_moe_product_bf16(_p(out), _DT[out_dtype], _p(a), _p(w), _p(order), _p(seg), E, top, 1 if gather else 0,
+                                              P, N, Kk, a.stride(0), 1 if relu2 else 0, ctypes.c_float(scale), form, _stream())
+        if code != -2:
+            _check(code, "moe_product")
+            return out
     _check(_lib().llogos_moe_product(_p(out), _DT[out_dtype], _p(a), _dt(a), _p(w), _dt(w), _p(order), _p(seg), E, top,
                                      1 if gather else 0, P, N, Kk, a.stride(0), 1 if relu2 else 0, ctypes.c_float(scale), _stream()),
            "moe_product")

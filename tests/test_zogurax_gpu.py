@@ -255,10 +255,15 @@ def test_a_far_key_the_unit_and_the_bend_decide_in_the_attention_alone():
         assert np.abs(np.concatenate(got) - want).max() <= PART_TOL[dtype] * size * (1 if dtype == "float32" else 2)
 
 
-@pytest.mark.parametrize("dtype", H.DTYPES)
+@pytest.mark.parametrize("dtype,form", [("float32", "auto"), ("bfloat16", "auto"), ("bfloat16", "plain"), ("bfloat16", "few"),
+                                        ("bfloat16", "tiles64"), ("bfloat16", "tiles128")])
 @pytest.mark.parametrize("experts,top,ff,shared,hidden,T", [(5, 2, 40, 24, 96, 9), (1, 1, 16, 8, 32, 3), (4, 4, 24, 0, 48, 70),
-                                                           (7, 3, 72, 136, 64, 300), (16, 1, 96, 96, 128, 1)])
-def test_the_experts_by_table(dtype, experts, top, ff, shared, hidden, T):
+                                                           (7, 3, 72, 136, 64, 300), (16, 1, 96, 96, 128, 1), (3, 2, 132, 20, 200, 150),
+                                                           (2, 1, 30, 6, 36, 40)])
+def test_the_experts_by_table(dtype, form, experts, top, ff, shared, hidden, T, monkeypatch):
+    """Every form of the experts' product (chosen by the step, or forced: plain multiply-adds, and on the matrix
+    cores tiles of 16, 64 and 128 sorted rows); the last shape has a width that only the plain form takes."""
+    monkeypatch.setattr(K, "MOE_PRODUCT", form)
     rng = np.random.default_rng(experts * 10 + top)
     vocab = 37
     moe = P.TableMoE(prefix="f.", hidden=hidden, vocab=vocab, n_experts=experts, top=top, intermediate=ff, shared_intermediate=shared)
