@@ -175,15 +175,16 @@ def zogurax_config(width, runs, vocab, ff):
             "torch_dtype": "bfloat16"}
 
 
-def moe_bytes_read(model, rows: int) -> int:
-    """Bytes of weights that a step of `rows` tokens reads at most: as step_weight_bytes, but of a layer's experts
-    only as many as the rows can choose."""
+def moe_bytes_read(model, ids) -> int:
+    """Bytes of weights that a step with the token ids `ids` reads: as step_weight_bytes, but of a layer's experts
+    only those that the layer's table names for these ids."""
     total = model.step_weight_bytes()
     for e in model.schedule:
         for f in model.layers[e.layer].feed_forwards():
             if hasattr(f, "n_experts"):
                 experts = (f.up.numel() + f.down.numel()) * f.up.element_size()
-                total -= experts - experts * min(f.n_experts, rows * f.top) // f.n_experts
+                chosen = len(set(f.table[list(ids)].reshape(-1).tolist()))
+                total -= experts - experts * chosen // f.n_experts
     return total
 
 
@@ -233,18 +234,19 @@ def compare_designs(args) -> int:
         for batch in (1, 8):
             slots = [eng.alloc_slot() for _ in range(batch)]
             eng.step([(x, toks(args.prompt_len)) for x in slots], want="last")
-            step = lambda: eng.step([(x, [1]) for x in slots], want="last", borrow=True)
+            ids = toks(batch)                                     # a token of its own for every sequence (an expert choice of its own)
+            step = lambda: eng.step([(x, [t]) for x, t in zip(slots, ids)], want="last", borrow=True)
             for _ in range(args.warmup):
                 step()
             dt = timed(lambda: [step() for _ in range(args.steps)], repeat=2) / args.steps
             out[f"decode_b{batch}_tok_s"] = round(batch / dt)
             out[f"decode_b{batch}_us"] = round(dt * 1e6, 1)
-            out[f"decode_b{batch}_roofline"] = round(moe_bytes_read(model, batch) / HBM_PEAK / dt, 3)
+            out[f"decode_b{batch}_roofline"] = round(moe_bytes_read(model, ids) / HBM_PEAK / dt, 3)
             if batch == 8:
                 probe = llogos.StepProbe()
                 probe.hold()
                 probe.start()
-                eng.step([(x, [1]) for x in slots], want="last", probe=probe)
+                eng.step([(x, [t]) for x, t in zip(slots, ids)], want="last", probe=probe)
                 out["decode_b8_parts_us"] = {k: round(v, 1) for k, v in probe.microseconds_per_call().items()}
             for x in slots:
                 eng.free_slot(x)

@@ -22,26 +22,29 @@ template <bool MASKED, int VP>
 __device__ __forceinline__ void softmax_page_bent(f32x4 (&s)[4], WaveState<VP>& st, float scale, float cap, int q_pos,
                                                   int key0, bf16x8 (&pf)[2], float& corr) {
     const int g = (threadIdx.x & (kWave - 1)) >> 4;
-    const float two_over_cap_log2 = cap > 0.f ? 2.0f * kLog2e / cap : 0.f;
     float y[16];
+    if (cap > 0.f) {
+        // cap * tanh(x / cap) * log2(e) = a - 2 a / (exp2(s * b) + 1) with a = cap * log2(e), b = 2 scale log2(e) / cap
+        const float a = cap * kLog2e, b2 = 2.0f * scale * kLog2e / cap;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const float t = __builtin_amdgcn_exp2f(s[i >> 2][i & 3] * b2);
+            y[i] = fmaf(-2.0f * a, __builtin_amdgcn_rcpf(t + 1.0f), a);
+        }
+    } else {
+        const float b1 = scale * kLog2e;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) y[i] = s[i >> 2][i & 3] * b1;
+    }
     float tile_max = -INFINITY;
 #pragma unroll
-    for (int rb = 0; rb < 4; ++rb)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            float x = s[rb][r] * scale;
-            if (cap > 0.f) {
-                const float t = __builtin_amdgcn_exp2f(x * two_over_cap_log2);
-                x = cap * (1.0f - 2.0f * __builtin_amdgcn_rcpf(t + 1.0f));
-            }
-            x *= kLog2e;
-            if (MASKED) {
-                const int key = key0 + g * 16 + rb * 4 + r;
-                if (!(q_pos >= 0 && key <= q_pos)) x = -INFINITY;
-            }
-            y[4 * rb + r] = x;
-            tile_max = fmaxf(tile_max, x);
+    for (int i = 0; i < 16; ++i) {
+        if (MASKED) {
+            const int key = key0 + g * 16 + i;                 // (i = 4 rb + r: the lane's keys are 16 in a row)
+            if (!(q_pos >= 0 && key <= q_pos)) y[i] = -INFINITY;
         }
+        tile_max = fmaxf(tile_max, y[i]);
+    }
     tile_max = quad_max(tile_max);
     const float m_new = fmaxf(st.m, tile_max);
     const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
@@ -80,6 +83,27 @@ __device__ __forceinline__ void attend_page_kv(WaveState<VP>& st, const bf16x8 (
     if (all_visible) softmax_page_bent<false, VP>(s, st, scale, cap, q_pos, key0, pf, corr);
     else             softmax_page_bent<true, VP>(s, st, scale, cap, q_pos, key0, pf, corr);
     weigh_values<VP>(st, vf, pf, corr, valid_keys);
+}
+
+// Fragment loads that may stay in the caches: a prompt's four waves of a block, and the blocks of the other
+// heads of a kv head, ask for the same pages at about the same time.
+template <int KP>
+__device__ __forceinline__ void load_keys_kept(bf16x8 (&kf)[4][KP / 32], const bf16_t* __restrict__ kpage) {
+    const bf16_t* mine = kpage + 8 * (threadIdx.x & (kWave - 1));
+#pragma unroll
+    for (int rb = 0; rb < 4; ++rb)
+#pragma unroll
+        for (int sk = 0; sk < KP / 32; ++sk) kf[rb][sk] = ld_frag(mine + 512 * (rb * (KP / 32) + sk));
+}
+
+template <int VP>
+__device__ __forceinline__ void load_values_kept(bf16x8 (&vf)[VP / 16][2], const bf16_t* __restrict__ vpage) {
+    const bf16_t* mine = vpage + 8 * (threadIdx.x & (kWave - 1));
+#pragma unroll
+    for (int db = 0; db < VP / 16; ++db) {
+        vf[db][0] = ld_frag(mine + 512 * (2 * db));
+        vf[db][1] = ld_frag(mine + 512 * (2 * db + 1));
+    }
 }
 
 // What finishes a row: the sink's share of the denominator (exp(0 - max), the maximum being in units of
@@ -129,11 +153,27 @@ __global__ __launch_bounds__(kAttnWaves * kWave) void capped_prefill_kernel(
     WaveState<VP> st;
     st.init();
     const int n_pages = last_pos / kPageTokens + 1;
+    // The next page's keys are asked for as soon as this page's scores are taken (their registers are free then),
+    // behind this page's values: the softmax and the second product cover their way.
+    auto page_of = [&](int pi) { return ((size_t)table[(size_t)b * table_stride + pi] * n_kv_heads + kvh) * kPageTokens; };
+    bf16x8 kf[4][KS];
+    size_t page = page_of(0);
+    load_keys_kept<KP>(kf, k_pool + page * KP);
     for (int pi = 0; pi < n_pages; ++pi) {
         const int key0 = pi * kPageTokens;
-        const size_t page = ((size_t)table[(size_t)b * table_stride + pi] * n_kv_heads + kvh) * kPageTokens;
-        attend_page_kv<KP, VP>(st, qf, k_pool + page * KP, v_pool + page * VP, q_pos, key0, min(kPageTokens, written - key0),
-                               rows == 16 && key0 + kPageTokens - 1 <= first_pos, scale, cap);
+        f32x4 s[4];
+        page_scores<KP>(s, kf, qf);
+        bf16x8 vf[VB][2];
+        load_values_kept<VP>(vf, v_pool + page * VP);
+        if (pi + 1 < n_pages) {
+            page = page_of(pi + 1);
+            load_keys_kept<KP>(kf, k_pool + page * KP);
+        }
+        bf16x8 pf[2];
+        float corr;
+        if (rows == 16 && key0 + kPageTokens - 1 <= first_pos) softmax_page_bent<false, VP>(s, st, scale, cap, q_pos, key0, pf, corr);
+        else                                                   softmax_page_bent<true, VP>(s, st, scale, cap, q_pos, key0, pf, corr);
+        weigh_values<VP>(st, vf, pf, corr, min(kPageTokens, written - key0));
     }
     if (!col_ok) return;
     const float f = finish_factor(st.m, st.l, unit_sink, gate ? gate + (size_t)my_row * gate_stride + h : nullptr);
@@ -280,7 +320,8 @@ static int capped_pages_per_wave(int batch, int n_kv_heads, int table_width) {
     else if (dk == 96 && dv == 96) DO(3, 6); else if (dk == 96 && dv == 128) DO(3, 8); else if (dk == 128 && dv == 64) DO(4, 4); \
     else if (dk == 128 && dv == 80) DO(4, 5); else if (dk == 128 && dv == 96) DO(4, 6); else DO(4, 8);
 
-// -2: a shape these kernels do not take (the caller uses the kernel for any shape)
+// -2: a shape these kernels do not take (the caller uses the kernel for any shape).  n_tiles counts tiles of 64
+// rows over all sequences.
 LLOGOS_EXPORT int llogos_capped_attn_prefill_bf16(void* out, const void* q, int q_stride, const void* k_pool, const void* v_pool,
                                                   const int* table, int table_stride, const int* cu, const int* tok_pos,
                                                   int batch, int n_tiles, int n_heads, int n_kv_heads, int dk, int dv, float scale,

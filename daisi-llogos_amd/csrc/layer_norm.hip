@@ -92,6 +92,10 @@ LLOGOS_EXPORT int llogos_layernorm(void* out, int out_dtype, float* x, const voi
     if (R <= 0 || H <= 0 || parts < 1) return LLOGOS_BAD_ARGUMENT;
     // as many threads as give each at most kLnItems values, in whole waves, 64 to 1024
     int threads = H <= 256 ? 64 : (H <= 1024 ? 128 : (H <= 4096 ? 256 : 1024));
+    if (R <= 64) {                       // few rows: four values a thread, so that a row's loads are all in flight at once
+        threads = ((H + 3) / 4 + kWave - 1) / kWave * kWave;
+        threads = threads < 64 ? 64 : (threads > 1024 ? 1024 : threads);
+    }
     const bool cached = (size_t)threads * kLnItems >= (size_t)H;
 #define LN(TO, TD) do { \
         if (cached) layernorm_kernel<TO, TD, true><<<R, threads, 0, stream>>>((TO*)out, x, (const TD*)delta, parts, (size_t)part_stride, rows, w, eps, H, write_back); \

@@ -13,7 +13,7 @@
 #include "common.h"
 
 template <typename T>
-__global__ __launch_bounds__(256) void qkv_prepare_kernel(
+__global__ __launch_bounds__(1024) void qkv_prepare_kernel(
         const float* __restrict__ qkv, int parts, size_t part_stride, int row_stride, const float* __restrict__ bias,
         T* __restrict__ q_out, int n_heads, int n_kv_heads, int head_dim, int v_dim, int k_page_dim, int v_page_dim,
         const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w, float eps, float temp_coef, int temp_every,
@@ -83,7 +83,9 @@ LLOGOS_EXPORT int llogos_qkv_prepare(const float* qkv, int parts, long long part
         if (k_page_dim < head_dim || v_page_dim < v_dim || (k_page_dim % 8) || (v_page_dim % 16)) return LLOGOS_BAD_ARGUMENT;
     }
     if (row_stride < n_heads * head_dim + n_kv_heads * (head_dim + v_dim)) return LLOGOS_BAD_ARGUMENT;
-#define PREP(T_) qkv_prepare_kernel<T_><<<T, 256, 0, stream>>>(qkv, parts, (size_t)part_stride, row_stride, bias, (T_*)q_out, \
+    // few rows: many threads a row, so that a row's loads are all in flight at once
+    const int threads = T <= 64 ? 1024 : 256;
+#define PREP(T_) qkv_prepare_kernel<T_><<<T, threads, 0, stream>>>(qkv, parts, (size_t)part_stride, row_stride, bias, (T_*)q_out, \
         n_heads, n_kv_heads, head_dim, v_dim, k_page_dim, v_page_dim, q_norm_w, k_norm_w, eps, temp_coef, temp_every, \
         (T_*)k_pool, (T_*)v_pool, table, table_stride, tok_seq, tok_pos)
     if (dtype == DT_F32) PREP(float);
