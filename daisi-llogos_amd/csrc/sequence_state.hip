@@ -19,8 +19,10 @@ template <typename TO>
 __global__ void causal_conv_kernel(TO* __restrict__ out, const float* __restrict__ h, const float* __restrict__ w,
                                    float* __restrict__ state, const int* __restrict__ slots,
                                    const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
-                                   const int* __restrict__ cu, int W, int ldh, int taps, int update_state, int add_input) {
-    const int t = blockIdx.x;
+                                   const int* __restrict__ cu, int W, int ldh, int taps, int update_state, int add_input,
+                                   int T, int per_block) {
+  // a block takes per_block tokens in turn (a long step's blocks are otherwise too short to hide their loads)
+  for (int t = blockIdx.x * per_block; t < min(T, (int)(blockIdx.x + 1) * per_block); ++t) {
     const int seq = tok_seq[t], pos = tok_pos[t];
     const int before = cu ? t - cu[seq] : 0;                 // tokens of this sequence earlier in the step
     float* st = state + (size_t)slots[seq] * (taps - 1) * W;
@@ -46,6 +48,7 @@ __global__ void causal_conv_kernel(TO* __restrict__ out, const float* __restrict
                 if (j < taps) st[(size_t)(taps - 1 - j) * W + c] = (j == 1) ? x0 : old[j - 1];
         }
     }
+  }
 }
 
 // The state after a step of any length: row i <- the input at position new_len - (taps - 1) + i,
@@ -78,12 +81,13 @@ LLOGOS_EXPORT int llogos_causal_conv(void* out, int out_dtype, const float* h, c
     if (!cu && T != B) return LLOGOS_BAD_ARGUMENT;
     const int threads = 256;
     const int by = (W + threads - 1) / threads;
-    dim3 grid(T, by);
+    const int per_block = T > 512 ? 8 : 1;
+    dim3 grid((T + per_block - 1) / per_block, by);
     const int fused = cu ? 0 : 1;
     if (out_dtype == DT_F32)
-        causal_conv_kernel<float><<<grid, threads, 0, stream>>>((float*)out, h, w, state, slots, tok_seq, tok_pos, cu, W, ldh, taps, fused, add_input);
+        causal_conv_kernel<float><<<grid, threads, 0, stream>>>((float*)out, h, w, state, slots, tok_seq, tok_pos, cu, W, ldh, taps, fused, add_input, T, per_block);
     else if (out_dtype == DT_BF16)
-        causal_conv_kernel<bf16_t><<<grid, threads, 0, stream>>>((bf16_t*)out, h, w, state, slots, tok_seq, tok_pos, cu, W, ldh, taps, fused, add_input);
+        causal_conv_kernel<bf16_t><<<grid, threads, 0, stream>>>((bf16_t*)out, h, w, state, slots, tok_seq, tok_pos, cu, W, ldh, taps, fused, add_input, T, per_block);
     else
         return LLOGOS_BAD_ARGUMENT;
     if (cu && taps > 1) conv_state_kernel<<<dim3(B, by), threads, 0, stream>>>(h, state, slots, cu, W, ldh, taps);

@@ -118,11 +118,14 @@ def test_the_position_vector_is_added(width):
     assert np.abs(_np(x) - 2.0 - pz.position_vector(pos, width)).max() <= 2e-7
 
 
+@pytest.mark.parametrize("lengths,cuts", [((19, 6, 1), [(5, 2, 1), (1, 1, 0), (1, 1, 0), (2, 2, 0), (1, 0, 0), (9, 0, 0)]),
+                                          ((700, 30, 2), [(640, 29, 1), (1, 1, 1), (59, 0, 0)])])
 @pytest.mark.parametrize("taps", [1, 2, 4])
-def test_the_convolution_behind_a_projection_over_steps_of_any_size(taps):
-    """Without its input added, on the first columns of wider rows, with the projected rows as state."""
+def test_the_convolution_behind_a_projection_over_steps_of_any_size(taps, lengths, cuts):
+    """Without its input added, on the first columns of wider rows, with the projected rows as state; a long
+    step's blocks take several tokens each."""
     rng = np.random.default_rng(taps)
-    W, wide, lengths = 70, 77, (19, 6, 1)
+    W, wide = 70, 77
     w = rng.uniform(-0.8, 0.8, size=(W, taps))
     h = [rng.standard_normal((n, wide)).astype(np.float32) for n in lengths]
     want = [pz.time_convolution(x[:, :W], w) for x in h]
@@ -130,7 +133,7 @@ def test_the_convolution_behind_a_projection_over_steps_of_any_size(taps):
     state = torch.zeros((5, taps - 1, W), dtype=torch.float32, device=DEV)
     got = [np.zeros((n, W)) for n in lengths]
     rt = P.Runtime(DEV, torch.float32)
-    for seqs, lo, hi in _steps(lengths, [(5, 2, 1), (1, 1, 0), (1, 1, 0), (2, 2, 0), (1, 0, 0), (9, 0, 0)]):
+    for seqs, lo, hi in _steps(lengths, cuts):
         ctx = _ctx(rt, hi, [b - a for a, b in zip(lo, hi)], [slots[i] for i in seqs])
         rows = torch.tensor(np.concatenate([h[i][a:b] for i, a, b in zip(seqs, lo, hi)]), device=DEV)
         o = _np(K.causal_conv(ctx, rows[:, :W], torch.tensor(w, dtype=torch.float32, device=DEV), state, torch.float32, add_input=False))
