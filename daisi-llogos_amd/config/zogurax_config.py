@@ -28,7 +28,7 @@ class ZoguraxMixerConfig:
     softcap: float      # 0: scores are not bent
     temp_coef: float    # 0: no factor on the query
     temp_every: int
-    conv: int           # taps of the convolution behind the projections ('attention' only)
+    conv: int           # taps of the convolution behind the projections ('attention' only; 0: none)
 
 
 @dataclass(frozen=True)
@@ -94,11 +94,11 @@ class ZoguraxConfig:
             heads = mr.int("heads")
             mixer = ZoguraxMixerConfig(heads, mr.int("kv_heads", heads), mr.int("dim"), mr.int("vdim"), mr.float("scale"),
                                        mr.float("softcap", 0.0), coef, every,
-                                       mr.int("conv") if kind == "attention" else 0)
+                                       mr.int("conv", 0) if kind == "attention" else 0)
             if min(mixer.heads, mixer.kv_heads, mixer.dim, mixer.vdim) <= 0 or mixer.heads % mixer.kv_heads:
                 raise ConfigError(f"{where}.mixer: heads, kv_heads, dim and vdim must be positive, heads a multiple of kv_heads")
-            if mixer.softcap < 0 or (kind == "attention" and mixer.conv < 1):
-                raise ConfigError(f"{where}.mixer: softcap must not be negative and conv must be at least 1")
+            if mixer.softcap < 0 or mixer.conv < 0:
+                raise ConfigError(f"{where}.mixer: softcap and conv must not be negative")
             mlp = lr.obj("mlp", None)
             if mlp is not None:
                 fr = ConfigReader(mlp, where + ".mlp")

@@ -118,7 +118,7 @@ __device__ __forceinline__ float finish_factor(float m, float l, int unit_sink, 
 // ---------------------------------------------------------------- prefill
 // grid (tiles of 64 tokens over all sequences, heads); wave w takes rows 16 w .. 16 w + 15 of the tile.
 template <int KS, int VB>
-__global__ __launch_bounds__(kAttnWaves * kWave) void capped_prefill_kernel(
+__global__ __launch_bounds__(kAttnWaves * kWave) __attribute__((amdgpu_waves_per_eu(2, 2))) void capped_prefill_kernel(
         bf16_t* __restrict__ out, const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_pool,
         const bf16_t* __restrict__ v_pool, const int* __restrict__ table, int table_stride, const int* __restrict__ cu,
         const int* __restrict__ tok_pos, int batch, int n_heads, int n_kv_heads, int group, float scale, float cap,

@@ -282,7 +282,7 @@ __global__ __launch_bounds__(256) void moe_few_kernel(TO* __restrict__ out, cons
 constexpr int kMoeBN = 128, kMoeBK = 64, kMoeLd = 80;      // LDS rows of 64 values, 160 bytes apart
 
 template <int BM, typename TO>
-__global__ __launch_bounds__(256) void moe_tiles_kernel(TO* __restrict__ out, const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void moe_tiles_kernel(TO* __restrict__ out, const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
                                                         const int* __restrict__ order, const int* __restrict__ seg, int E, int top,
                                                         int gather, int N, int K, int lda, int act, float scale) {
     constexpr int CA = BM * 8 / 256, CW = kMoeBN * 8 / 256;           // 16-byte pieces a thread copies a stage

@@ -37,7 +37,7 @@ def test_the_reader_takes_every_size_and_constant_from_the_file():
 
 
 @pytest.mark.parametrize("path,value,word", [
-    (("layers", 0, "type"), "attention_3", "attention_3"), (("layers", 1, "mixer", "conv"), None, "conv"),
+    (("layers", 0, "type"), "attention_3", "attention_3"), (("layers", 1, "mixer", "conv"), -1, "conv"),
     (("layers", 0, "mixer", "kv_heads"), 3, "kv_heads"), (("layers", 0, "mlp", "kind"), "dense", "dense"),
     (("layers", 0, "mlp", "router", "top"), 9, "top"), (("loop", "stop"), 7, "loop"), (("loop", "times"), 0, "loop"),
     (("layers", 0, "mixer", "q_temp", "every"), 0, "every"), (("norm",), None, "norm"), (("width",), "wide", "width")])
