@@ -204,8 +204,8 @@ LLOGOS_EXPORT int llogos_moe_combine(float* out, const float* y, const int* wher
 //   few rows  tiles of 16 sorted rows; a block of four waves owns 16 rows of the matrix, its waves take the
 //             steps of 32 k in turn (together whole cache lines), straight from memory into operands, and LDS
 //             adds the four waves' sums in order;
-//   tiles     64 or 128 sorted rows x 128 rows of the matrix, stages of 64 k through LDS (rows 160 bytes
-//             apart: fragment reads without bank conflicts), the next stage's loads in registers meanwhile.
+//   tiles     64 or 128 sorted rows x 128 rows of the matrix with v_mfma_f32_32x32x16_bf16, stages of 64 k
+//             through LDS (swizzled rows of 128 bytes), the next stage's loads in registers meanwhile.
 // Sums depend on k's order alone, as above.  K must be a multiple of 8 and N of 4.
 typedef __bf16 moe_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float moe_f32x4 __attribute__((ext_vector_type(4)));
@@ -279,16 +279,24 @@ __global__ __launch_bounds__(256) void moe_few_kernel(TO* __restrict__ out, cons
     if (m < m_end && n < N) moe_store4(out + (size_t)m * N + n, v[0], v[1], v[2], v[3]);
 }
 
-constexpr int kMoeBN = 128, kMoeBK = 64, kMoeLd = 80;      // LDS rows of 64 values, 160 bytes apart
+constexpr int kMoeBK = 64;      // LDS rows of 64 values of k: 128 bytes, eight pieces of 16
+typedef float moe_f32x16 __attribute__((ext_vector_type(16)));
 
-template <int BM, typename TO>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void moe_tiles_kernel(TO* __restrict__ out, const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
-                                                        const int* __restrict__ order, const int* __restrict__ seg, int E, int top,
-                                                        int gather, int N, int K, int lda, int act, float scale) {
-    constexpr int CA = BM * 8 / 256, CW = kMoeBN * 8 / 256;           // 16-byte pieces a thread copies a stage
-    constexpr int WN = BM == 128 ? 64 : 32, NT = WN / 16, MT = 4;     // a wave's part: 64 rows x WN columns of the tile
-    __shared__ __attribute__((aligned(16))) bf16_t As[BM * kMoeLd];
-    __shared__ __attribute__((aligned(16))) bf16_t Ws[kMoeBN * kMoeLd];
+// where piece `oct` (8 values of k) of row `row` lies in an LDS tile: the eight pieces of a row are swizzled so
+// that the 32 rows an operand read touches spread over all banks
+__device__ __forceinline__ int moe_lds_at(int row, int oct) { return row * kMoeBK + ((oct ^ ((row >> 1) & 7)) << 3); }
+
+// v_mfma_f32_32x32x16_bf16: an operand is 32 rows x 16 k, lane l holding row l & 31 and k 8 (l >> 5) .. + 7; the
+// rows of the expert's matrix are the first operand and the sorted rows the second, so a lane ends with the sums
+// of one sorted row (l & 31) for 4 x 4 neighbouring columns: entry 4 q + e is column 8 q + 4 (l >> 5) + e.
+template <int BM, int BN, typename TO>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void moe_tiles_kernel(
+        TO* __restrict__ out, const bf16_t* __restrict__ a, const bf16_t* __restrict__ w, const int* __restrict__ order,
+        const int* __restrict__ seg, int E, int top, int gather, int N, int K, int lda, int act, float scale) {
+    constexpr int CA = BM * 8 / 256, CW = BN * 8 / 256;           // 16-byte pieces a thread copies a stage
+    constexpr int WN = BM == 128 ? BN / 2 : BN / 4, NT = WN / 32, MT = 2;     // a wave's part: 64 rows x WN columns of the tile
+    __shared__ __attribute__((aligned(16))) bf16_t As[BM * kMoeBK];
+    __shared__ __attribute__((aligned(16))) bf16_t Ws[BN * kMoeBK];
     __shared__ int src_row[BM];
     __shared__ int s_tile[3];
     const int tid = threadIdx.x;
@@ -302,24 +310,26 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     }
     __syncthreads();
     const int lane = tid & (kWave - 1), wave = tid / kWave;
-    const int c = lane & 15, g = lane >> 4;
+    const int r32 = lane & 31, h = lane >> 5;
     const int wm = BM == 128 ? wave >> 1 : 0, wn = BM == 128 ? wave & 1 : wave;
-    const int n0 = blockIdx.x * kMoeBN;
+    const int n0 = blockIdx.x * BN;
     const bf16_t* we = w + (size_t)e * N * K;
 
     const bf16_t* pa[CA];
     const bf16_t* pw[CW];
-    int ka[CA], kw[CW];
+    int ka[CA], kw[CW], la[CA], lw[CW];
 #pragma unroll
     for (int j = 0; j < CA; ++j) {
         const int q = tid + 256 * j, row = q >> 3;
         ka[j] = (q & 7) * 8;
+        la[j] = moe_lds_at(row, q & 7);
         pa[j] = src_row[row] >= 0 ? a + (size_t)src_row[row] * lda + ka[j] : nullptr;
     }
 #pragma unroll
     for (int j = 0; j < CW; ++j) {
         const int q = tid + 256 * j, row = q >> 3;
         kw[j] = (q & 7) * 8;
+        lw[j] = moe_lds_at(row, q & 7);
         pw[j] = n0 + row < N ? we + (size_t)(n0 + row) * K + kw[j] : nullptr;
     }
     uint4 ra[CA], rw[CW];
@@ -331,58 +341,56 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
         for (int j = 0; j < CW; ++j)
             rw[j] = (pw[j] && k0 + kw[j] < K) ? *reinterpret_cast<const uint4*>(pw[j] + k0) : make_uint4(0, 0, 0, 0);
     };
-    moe_f32x4 acc[NT][MT];
+    moe_f32x16 acc[NT][MT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = moe_f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[nt][mt][v] = 0.f;
 
     fetch(0);
     for (int k0 = 0; k0 < K; k0 += kMoeBK) {
 #pragma unroll
-        for (int j = 0; j < CA; ++j) {
-            const int q = tid + 256 * j;
-            *reinterpret_cast<uint4*>(As + (q >> 3) * kMoeLd + (q & 7) * 8) = ra[j];
-        }
+        for (int j = 0; j < CA; ++j) *reinterpret_cast<uint4*>(As + la[j]) = ra[j];
 #pragma unroll
-        for (int j = 0; j < CW; ++j) {
-            const int q = tid + 256 * j;
-            *reinterpret_cast<uint4*>(Ws + (q >> 3) * kMoeLd + (q & 7) * 8) = rw[j];
-        }
+        for (int j = 0; j < CW; ++j) *reinterpret_cast<uint4*>(Ws + lw[j]) = rw[j];
         __syncthreads();
         if (k0 + kMoeBK < K) fetch(k0 + kMoeBK);
 #pragma unroll
-        for (int ks = 0; ks < kMoeBK / 32; ++ks) {
+        for (int ks = 0; ks < kMoeBK / 16; ++ks) {
             moe_bf16x8 af[MT], wf[NT];
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) af[mt] = moe_frag(As + (wm * 64 + mt * 16 + c) * kMoeLd + ks * 32 + 8 * g);
+            for (int mt = 0; mt < MT; ++mt) af[mt] = moe_frag(As + moe_lds_at(wm * 64 + mt * 32 + r32, 2 * ks + h));
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) wf[nt] = moe_frag(Ws + (wn * WN + nt * 16 + c) * kMoeLd + ks * 32 + 8 * g);
+            for (int nt = 0; nt < NT; ++nt) wf[nt] = moe_frag(Ws + moe_lds_at(wn * WN + nt * 32 + r32, 2 * ks + h));
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt)
-                    acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[nt], af[mt], acc[nt][mt], 0, 0, 0);
+                    acc[nt][mt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[nt], af[mt], acc[nt][mt], 0, 0, 0);
         }
         __syncthreads();
     }
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-        const int m = m0 + wm * 64 + mt * 16 + c;
+        const int m = m0 + wm * 64 + mt * 32 + r32;
         if (m >= m_end) continue;
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-            const int n = n0 + wn * WN + nt * 16 + 4 * g;
-            if (n >= N) continue;
-            float v[4];
+        for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                v[r] = acc[nt][mt][r];
-                if (act == 1) { v[r] = fmaxf(v[r], 0.f); v[r] *= v[r]; }
-                v[r] *= scale;
+            for (int q = 0; q < 4; ++q) {
+                const int n = n0 + wn * WN + nt * 32 + 8 * q + 4 * h;
+                if (n >= N) continue;
+                float v[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    v[r] = acc[nt][mt][4 * q + r];
+                    if (act == 1) { v[r] = fmaxf(v[r], 0.f); v[r] *= v[r]; }
+                    v[r] *= scale;
+                }
+                moe_store4(out + (size_t)m * N + n, v[0], v[1], v[2], v[3]);
             }
-            moe_store4(out + (size_t)m * N + n, v[0], v[1], v[2], v[3]);
-        }
     }
 }
 
@@ -398,8 +406,8 @@ LLOGOS_EXPORT int llogos_moe_product_bf16(void* out, int out_dtype, const void* 
 #define MOE_GO(KERNEL, NB, TO) KERNEL<<<dim3((N + NB - 1) / NB, row_tiles), 256, 0, stream>>>((TO*)out, (const bf16_t*)a, (const bf16_t*)w, \
         order, seg, E, top, gather, N, K, lda, act, scale)
     if (form == 0) { if (out_dtype == DT_F32) MOE_GO(moe_few_kernel<float>, 16, float); else MOE_GO(moe_few_kernel<bf16_t>, 16, bf16_t); }
-    else if (form == 1) { if (out_dtype == DT_F32) MOE_GO((moe_tiles_kernel<64, float>), kMoeBN, float); else MOE_GO((moe_tiles_kernel<64, bf16_t>), kMoeBN, bf16_t); }
-    else { if (out_dtype == DT_F32) MOE_GO((moe_tiles_kernel<128, float>), kMoeBN, float); else MOE_GO((moe_tiles_kernel<128, bf16_t>), kMoeBN, bf16_t); }
+    else if (form == 1) { if (out_dtype == DT_F32) MOE_GO((moe_tiles_kernel<64, 128, float>), 128, float); else MOE_GO((moe_tiles_kernel<64, 128, bf16_t>), 128, bf16_t); }
+    else { if (out_dtype == DT_F32) MOE_GO((moe_tiles_kernel<128, 128, float>), 128, float); else MOE_GO((moe_tiles_kernel<128, 128, bf16_t>), 128, bf16_t); }
 #undef MOE_GO
     return LLOGOS_LAUNCH_CHECK();
 }
