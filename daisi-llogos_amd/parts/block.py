@@ -9,6 +9,7 @@ steps of few rows, by the product that closes the mixer or the feed-forward, whi
 leaves the following norm's rows for the product that opens the next part."""
 from __future__ import annotations
 
+import os
 from typing import Callable, List, Optional, Tuple
 
 import torch
@@ -164,7 +165,16 @@ class ParallelBlock(Block):
 
     The feed-forward may be absent.  The mixer's output joins the stream at once (through its closing
     product where that can add itself, else by a sum kernel), the feed-forward's is handed on as `pending`;
-    without a feed-forward the mixer's output is."""
+    without a feed-forward the mixer's output is.
+
+    The two sublayers depend on the norm's rows alone, so in steps of few rows, whose kernels are short and
+    wait for one another, the feed-forward is queued on a second stream beside the mixer (also inside a
+    captured step, where the two become branches of the graph); both streams meet before the block returns.
+    Every use of the second stream begins by waiting for the first, after the norm that consumed what the
+    second stream made last, so memory that either stream's allocator hands out again is no longer read by
+    the other.  `LLOGOS_PARALLEL_STREAMS=0` keeps everything on one stream."""
+    side_rows = 0 if os.environ.get("LLOGOS_PARALLEL_STREAMS", "1") == "0" else 64     # steps of up to so many rows use the second stream
+    _side_streams = {}
 
     def __init__(self, mixer_norm: Norm, mixer: Mixer, ffn: Optional[FeedForward] = None):
         self.mixer_norm, self.mixer, self.ffn = mixer_norm, mixer, ffn
@@ -186,6 +196,15 @@ class ParallelBlock(Block):
         cache = caches[0] if isinstance(caches, (list, tuple)) else caches
         h = self.mixer_norm.forward(x, pending)
         mark(ctx, "norm")
+        d = side = None
+        if self.ffn is not None and h.shape[0] <= self.side_rows and (ctx is None or ctx.probe is None) and h.is_cuda:
+            main = torch.cuda.current_stream(h.device)
+            side = self._side_streams.get(h.device)
+            if side is None:
+                side = self._side_streams[h.device] = torch.cuda.Stream(device=h.device)
+            side.wait_stream(main)                       # the norm's rows are there
+            with torch.cuda.stream(side):
+                d = self.ffn.forward(ctx, h)
         if self.mixer.adds_to_residual:
             a = self.mixer.forward(ctx, h, cache, residual=Residual(x, None))
         else:
@@ -197,6 +216,9 @@ class ParallelBlock(Block):
             return x, a
         if a is not None:
             K.residual_add(x, K.sum_parts(a, None, torch.float32))
-        d = self.ffn.forward(ctx, h)
+        if side is not None:
+            torch.cuda.current_stream(h.device).wait_stream(side)
+        else:
+            d = self.ffn.forward(ctx, h)
         mark(ctx, "feed_forward")
         return x, d

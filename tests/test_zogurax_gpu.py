@@ -404,6 +404,28 @@ def test_long_decoding_replayed_and_launched(name, dtype):
     assert np.array_equal(outs[True], outs[False])              # a replayed step is the launched step
 
 
+@pytest.mark.parametrize("dtype", H.DTYPES)
+def test_the_feed_forward_on_a_second_stream_changes_no_bit(dtype, monkeypatch):
+    """Steps of few rows queue the feed-forward beside the mixer; with everything on one stream the same kernels
+    run one after the other.  Unequal batches, prompts of few rows and single tokens, replayed and launched."""
+    name = "zog_a"
+    seqs = [H.tokens(name, 40, 30 + i) for i in range(3)]
+    outs = {}
+    for rows in (64, 0):
+        monkeypatch.setattr(P.ParallelBlock, "side_rows", rows)
+        for graphs in (True, False):
+            eng = H.engine(name, dtype, use_graphs=graphs)
+            slots = [eng.alloc_slot() for _ in seqs]
+            got = [_np(eng.step([(s, list(t[:n])) for s, t, n in zip(slots, seqs, (20, 3, 9))], want="all"))]
+            for step in range(12):
+                got.append(_np(eng.step([(s, [t[n + step]]) for s, t, n in zip(slots, seqs, (20, 3, 9))], want="all")))
+            outs[(rows, graphs)] = np.concatenate(got)
+    first = outs[(64, True)]
+    assert all(np.array_equal(first, o) for o in outs.values())
+    want = np.concatenate([H.plain_logits(name, t)[:n] for t, n in zip(seqs, (20, 3, 9))])
+    H.close(first[:32], want, dtype, "two streams")
+
+
 def test_far_keys_the_unit_and_the_query_factor_decide_and_are_there():
     """On a sharpened model the logits of late positions depend on keys hundreds of positions back, on the
     unit in the denominator and on the query's factor by many times the bound; the engine agrees with the
