@@ -51,6 +51,71 @@ __global__ void causal_conv_kernel(TO* __restrict__ out, const float* __restrict
   }
 }
 
+// The same for steps of many tokens, four neighbouring channels a thread with 16-byte loads and stores (a thread's
+// loads are all asked for before the first sum): a long step is bound by how many requests its threads have in
+// flight, not by bytes.  For W, ldh multiples of 4 and 16-byte aligned rows; the state is not written here.
+__device__ __forceinline__ void conv_store4(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+__device__ __forceinline__ void conv_store4(bf16_t* p, float4 v) {
+    uint2 u;
+    u.x = (uint32_t)f32_to_bf16(v.x) | ((uint32_t)f32_to_bf16(v.y) << 16);
+    u.y = (uint32_t)f32_to_bf16(v.z) | ((uint32_t)f32_to_bf16(v.w) << 16);
+    *reinterpret_cast<uint2*>(p) = u;
+}
+
+constexpr int kConvWideTokens = 8;      // tokens a block of the wide kernel takes one after the other with its weights in LDS
+
+template <typename TO>
+__global__ void causal_conv_wide_kernel(TO* __restrict__ out, const float* __restrict__ h, const float* __restrict__ w,
+                                        const float* __restrict__ state, const int* __restrict__ slots,
+                                        const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
+                                        const int* __restrict__ cu, int T, int W, int ldh, int taps, int add_input) {
+    // the block's weights (4 * blockDim channels x taps, one run of memory) go through LDS: read channel by
+    // channel from memory they would cost a cache line a lane and load
+    extern __shared__ float wl[];
+    const int c0 = 4 * blockIdx.y * blockDim.x;
+    const int n_w = min(4 * (int)blockDim.x, W - c0) * taps;
+    for (int i = threadIdx.x; i < n_w; i += blockDim.x) wl[i] = w[(size_t)c0 * taps + i];
+    __syncthreads();
+    const int c = c0 + 4 * threadIdx.x;
+    if (c >= W) return;
+    const float* wc = wl + 4 * threadIdx.x * taps;
+    const int t_end = min(T, (int)(blockIdx.x + 1) * kConvWideTokens);
+#pragma unroll 2
+    for (int t = blockIdx.x * kConvWideTokens; t < t_end; ++t) {
+        const int seq = tok_seq[t], pos = tok_pos[t];
+        const int before = t - cu[seq];
+        const float* st = state + (size_t)slots[seq] * (taps - 1) * W;
+        float4 x[kMaxTaps];
+#pragma unroll
+        for (int j = 0; j < kMaxTaps; ++j) {
+            if (j < taps) {
+                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (j <= before) v = *reinterpret_cast<const float4*>(h + (size_t)(t - j) * ldh + c);
+                else if (pos - j >= 0) v = *reinterpret_cast<const float4*>(st + (size_t)(taps - 1 + before - j) * W + c);
+                x[j] = v;
+            }
+        }
+        // (the sums in the order of the one-channel kernel: the present token's product first, then the rows before it)
+        float4 acc;
+        acc.x = x[0].x * wc[0 * taps + taps - 1];
+        acc.y = x[0].y * wc[1 * taps + taps - 1];
+        acc.z = x[0].z * wc[2 * taps + taps - 1];
+        acc.w = x[0].w * wc[3 * taps + taps - 1];
+#pragma unroll
+        for (int j = 1; j < kMaxTaps; ++j) {
+            if (j < taps) {
+                const int k = taps - 1 - j;
+                acc.x = fmaf(wc[0 * taps + k], x[j].x, acc.x);
+                acc.y = fmaf(wc[1 * taps + k], x[j].y, acc.y);
+                acc.z = fmaf(wc[2 * taps + k], x[j].z, acc.z);
+                acc.w = fmaf(wc[3 * taps + k], x[j].w, acc.w);
+            }
+        }
+        if (add_input) { acc.x += x[0].x; acc.y += x[0].y; acc.z += x[0].z; acc.w += x[0].w; }
+        conv_store4(out + (size_t)t * W + c, acc);
+    }
+}
+
 // The state after a step of any length: row i <- the input at position new_len - (taps - 1) + i,
 // from this step's rows or from the old state.  A thread owns a channel of a sequence and
 // reads all it needs before it writes.
@@ -81,9 +146,24 @@ LLOGOS_EXPORT int llogos_causal_conv(void* out, int out_dtype, const float* h, c
     if (!cu && T != B) return LLOGOS_BAD_ARGUMENT;
     const int threads = 256;
     const int by = (W + threads - 1) / threads;
-    const int per_block = T > 512 ? 8 : 1;
+    const int per_block = 1;
     dim3 grid((T + per_block - 1) / per_block, by);
     const int fused = cu ? 0 : 1;
+    const bool wide = cu && T > 64 && (W % 4) == 0 && (ldh % 4) == 0 && ((uintptr_t)h % 16) == 0 && ((uintptr_t)out % 16) == 0 &&
+                      ((uintptr_t)state % 16) == 0;
+    if (wide) {
+        const int wthreads = 128;
+        dim3 wgrid((T + kConvWideTokens - 1) / kConvWideTokens, (W / 4 + wthreads - 1) / wthreads);
+        const size_t wlds = (size_t)wthreads * 4 * taps * sizeof(float);
+        if (out_dtype == DT_F32)
+            causal_conv_wide_kernel<float><<<wgrid, wthreads, wlds, stream>>>((float*)out, h, w, state, slots, tok_seq, tok_pos, cu, T, W, ldh, taps, add_input);
+        else if (out_dtype == DT_BF16)
+            causal_conv_wide_kernel<bf16_t><<<wgrid, wthreads, wlds, stream>>>((bf16_t*)out, h, w, state, slots, tok_seq, tok_pos, cu, T, W, ldh, taps, add_input);
+        else
+            return LLOGOS_BAD_ARGUMENT;
+        if (taps > 1) conv_state_kernel<<<dim3(B, by), threads, 0, stream>>>(h, state, slots, cu, W, ldh, taps);
+        return LLOGOS_LAUNCH_CHECK();
+    }
     if (out_dtype == DT_F32)
         causal_conv_kernel<float><<<grid, threads, 0, stream>>>((float*)out, h, w, state, slots, tok_seq, tok_pos, cu, W, ldh, taps, fused, add_input, T, per_block);
     else if (out_dtype == DT_BF16)
