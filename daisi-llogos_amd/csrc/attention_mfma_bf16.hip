@@ -315,280 +315,6 @@ __global__ __launch_bounds__(kAttnWaves * kWave) void attn_prefill_kernel(
     }
 }
 
-constexpr int kTileRows = 128;
-
-// ---------------------------------------------------------------- prefill, pages shared through LDS
-// grid: one block per (tile of 128 tokens over all sequences, head), in the order given in the
-// kernel; the 4 waves of a block take 32 rows each (two blocks of 16 columns) and walk the same
-// pages: a page is copied to LDS once per block (two buffers, the copy of the next page is in
-// flight while the current one is used), and every key and value fragment a wave reads serves
-// both of its column blocks.  A page's keys and values go from global memory into LDS without
-// passing through registers (16 bytes a lane, a wave's 64 lanes to 1 KB of consecutive LDS),
-// which frees the 32 registers of the copy and the time of the stores.  Pages are in fragment
-// order in memory, and so they are in LDS: a wave's read of a fragment is 64 x 16 consecutive
-// bytes, which LDS serves without a bank conflict; no padding and no swizzle.
-template <int HD>
-struct DirectPageLds {
-    bf16_t k[HD / 8][512];               // fragment (rb, sk) at rb * (HD / 32) + sk
-    bf16_t v[HD / 8][512];               // fragment (db, half) at 2 db + half
-};
-
-// HALVES = 2: a block of 8 waves, two sets of 4 with page buffers of their own, takes the same
-// 128 rows; the sets take the tile's pages in turn and add their results through LDS at the end.
-// One such block fills a compute unit (two waves a SIMD, as two blocks of 4 do), and a tile's
-// pages take half as long: with HALVES = 1 a block left alone on its unit goes no faster (one
-// wave a SIMD cannot overlap its matrix and its vector instructions), so a prompt of few tiles
-// took as long as the pages of its last tile, one after the other.
-template <int HD, int HALVES>
-__global__ __launch_bounds__(HALVES * kAttnWaves * kWave) __attribute__((amdgpu_waves_per_eu(2, 2)))
-void attn_prefill_direct_kernel(
-        bf16_t* __restrict__ out, const bf16_t* __restrict__ q, int q_stride,
-        const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
-        const int* __restrict__ table, int table_stride, const int* __restrict__ cu,
-        const int* __restrict__ tok_pos, int batch, int n_tiles, int n_heads, int n_kv_heads, int group,
-        float scale, int window, int sinks) {
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-    const int set = HALVES == 2 ? __builtin_amdgcn_readfirstlane(threadIdx.x / (kAttnWaves * kWave)) : 0;
-    DirectPageLds<HD>* lds = reinterpret_cast<DirectPageLds<HD>*>(smem_raw) + 2 * set;   // two buffers a set
-    // Blocks start in the order of their index, round-robin over the 8 XCDs.  Block L is the
-    // m-th block of XCD x (L = 8 m + x); an XCD takes the `group` query heads of one (tile, kv
-    // head) pair one after the other, so that the pair's pages stay in its L2, and the pairs go
-    // from the last tile to the first: late tiles of a causal prompt see the most keys, and
-    // starting with them keeps the compute units evenly busy to the end.
-    // A grid of at most two blocks per compute unit starts all at once, and the m-th and the
-    // (m + 32)-th block of an XCD share a compute unit: the second half runs in rising order
-    // then, so that the longest block shares with the shortest.
-    int m_xcd = blockIdx.x / 8;
-    const int xcd = blockIdx.x % 8, per_xcd = gridDim.x / 8;
-    if (HALVES == 1 && per_xcd > 32 && per_xcd <= 64 && m_xcd >= 32) m_xcd = per_xcd - 1 - (m_xcd - 32);
-    const int pair = (m_xcd / group) * 8 + xcd;
-    if (pair >= n_tiles * n_kv_heads) return;
-    const int kvh = pair % n_kv_heads, h = kvh * group + m_xcd % group;
-    int tile = n_tiles - 1 - pair / n_kv_heads, b = 0, first = 0;
-    for (; b < batch; ++b) {
-        const int len = cu[b + 1] - cu[b];
-        const int tiles = (len + kTileRows - 1) / kTileRows;
-        if (tile < tiles) { first = cu[b] + tile * kTileRows; break; }
-        tile -= tiles;
-    }
-    if (b >= batch) return;
-    const int lane = threadIdx.x & (kWave - 1);
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave) % kAttnWaves;   // within its set
-    const int c = lane & 15, g = lane >> 4;
-    const int seq_end = cu[b + 1];
-    const int tile_rows = min(kTileRows, seq_end - first);
-    const int tile_last_pos = tok_pos[first + tile_rows - 1];
-    const int tile_first_pos = tok_pos[first];
-    const int written = tok_pos[seq_end - 1] + 1;
-    const int row0 = first + 32 * wave;
-    const int wave_rows = max(0, min(32, seq_end - row0));
-    const bool ok0 = c < wave_rows, ok1 = 16 + c < wave_rows;
-    const int q_pos0 = ok0 ? tok_pos[row0 + c] : -1, q_pos1 = ok1 ? tok_pos[row0 + 16 + c] : -1;
-    bf16x8 qf0[HD / 32], qf1[HD / 32];
-    {
-        const bf16_t* qrow0 = q + (size_t)(row0 + (ok0 ? c : 0)) * q_stride + (size_t)h * HD + 8 * g;
-        const bf16_t* qrow1 = q + (size_t)(row0 + (ok1 ? 16 + c : 0)) * q_stride + (size_t)h * HD + 8 * g;
-#pragma unroll
-        for (int sk = 0; sk < HD / 32; ++sk) {
-            qf0[sk] = ok0 ? ld_frag(qrow0 + 32 * sk) : zero_frag();
-            qf1[sk] = ok1 ? ld_frag(qrow1 + 32 * sk) : zero_frag();
-        }
-    }
-    WaveState<HD> st0, st1;
-    st0.init();
-    st1.init();
-    const int wave_first_pos = wave_rows > 0 ? tok_pos[row0] : 0;
-    const int wave_last_pos = wave_rows > 0 ? tok_pos[row0 + wave_rows - 1] : -1;
-    const float scale_log2 = scale * kLog2e;
-
-    const int n_pages = tile_last_pos / kPageTokens + 1;
-    auto page_needed = [&](int pi) {
-        return page_may_be_visible_to_range(tile_first_pos, tile_last_pos, pi * kPageTokens, window, sinks);
-    };
-    auto next_needed = [&](int pi) {
-        ++pi;
-        while (pi < n_pages && !page_needed(pi)) ++pi;
-        return pi;
-    };
-    auto page_id = [&](int pi) { return table[(size_t)b * table_stride + pi]; };
-    auto page_base = [&](int id) { return ((size_t)id * n_kv_heads + kvh) * kPageTokens * HD; };
-    // This wave's share of a page's copy, in instructions of 1 KB (64 lanes x 16 bytes, a fragment):
-    // the block's instructions go to its waves in turn.
-    auto copy_page = [&](int id, DirectPageLds<HD>& pg) {
-        const bf16_t* kpage = k_pool + page_base(id);
-        const bf16_t* vpage = v_pool + page_base(id);
-#pragma unroll
-        for (int j = 0; j < HD / 8 / kAttnWaves; ++j) {
-            const int f = kAttnWaves * j + wave;
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(kpage + 512 * f + 8 * lane),
-                                             (__attribute__((address_space(3))) void*)&pg.k[f][0], 16, 0, 0);
-        }
-#pragma unroll
-        for (int j = 0; j < HD / 8 / kAttnWaves; ++j) {
-            const int f = kAttnWaves * j + wave;
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(vpage + 512 * f + 8 * lane),
-                                             (__attribute__((address_space(3))) void*)&pg.v[f][0], 16, 0, 0);
-        }
-    };
-    // The values of tokens that have not been written may be anything, also NaN, and 0 * NaN is
-    // NaN: in the one page of a sequence that is not full they are zeroed in LDS after the copy.
-    // Every lane does so with the pieces it copied itself, once they have arrived and before the
-    // block's barrier (one barrier a page, whatever the page: the two sets of HALVES = 2 are at
-    // different pages and must meet the same barriers).
-    auto zero_unwritten = [&](DirectPageLds<HD>& pg, int valid_keys) {
-#pragma unroll
-        for (int j = 0; j < HD / 8 / kAttnWaves; ++j) {
-            const int f = kAttnWaves * j + wave;
-            const int keep = valid_keys - 16 * (lane >> 4) - 8 * (f & 1);          // of the tokens this piece holds
-            if (keep >= 8) continue;
-            uint4* at = reinterpret_cast<uint4*>(&pg.v[f][8 * lane]);
-            *at = __builtin_bit_cast(uint4, keep_first(__builtin_bit_cast(bf16x8, *at), keep));
-        }
-    };
-    auto land = [&](int pi, DirectPageLds<HD>& pg) {                        // the copy of page pi is complete and visible
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        const int valid_keys = written - pi * kPageTokens;
-        if (pi < n_pages && valid_keys < kPageTokens) zero_unwritten(pg, valid_keys);
-        __syncthreads();
-    };
-    // The pages that are needed go to the sets in turn.  `lead` is the first set's page: every
-    // wave follows it, so that both sets go round the loop, and through its barriers, equally often.
-    auto advance = [&](int pi) {
-        pi = next_needed(pi);
-        return HALVES == 2 ? next_needed(pi) : pi;
-    };
-    int lead = next_needed(-1);
-    if (lead >= n_pages) return;                                         // cannot happen: a row sees itself
-    int cur = set ? next_needed(lead) : lead;
-    int nxt = advance(cur);
-    int nxt_id = nxt < n_pages ? page_id(nxt) : 0;
-    if (cur < n_pages) copy_page(page_id(cur), lds[0]);
-    land(cur, lds[0]);
-    int buf = 0;
-    while (lead < n_pages) {
-        const int nxt2 = advance(nxt);
-        if (nxt < n_pages) copy_page(nxt_id, lds[buf ^ 1]);
-        const int nxt2_id = nxt2 < n_pages ? page_id(nxt2) : 0;
-        do {
-        const int key0 = cur * kPageTokens;
-        if (cur >= n_pages) break;                                        // the second set, after an odd number of pages
-        if (wave_rows <= 0 || key0 > wave_last_pos) break;                // nothing of this page for this wave
-        if (!page_may_be_visible_to_range(wave_first_pos, wave_last_pos, key0, window, sinks)) break;
-        const DirectPageLds<HD>& pg = lds[buf];
-        f32x4 s0[4], s1[4];
-#pragma unroll
-        for (int rb = 0; rb < 4; ++rb) {
-            s0[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
-            s1[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
-        }
-#pragma unroll
-        for (int sk = 0; sk < HD / 32; ++sk) {
-#pragma unroll
-            for (int rb = 0; rb < 4; ++rb) {
-                const bf16x8 kf = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(
-                    &pg.k[rb * (HD / 32) + sk][8 * lane]));
-                s0[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf0[sk], s0[rb], 0, 0, 0);
-                s1[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf1[sk], s1[rb], 0, 0, 0);
-            }
-        }
-        auto read_v = [&](int db, int t) {
-            return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&pg.v[2 * db + t][8 * lane]));
-        };
-        constexpr int kEarly = 2;
-        bf16x8 vf[HD / 16][2];
-#pragma unroll
-        for (int db = 0; db < kEarly; ++db) { vf[db][0] = read_v(db, 0); vf[db][1] = read_v(db, 1); }
-        bf16x8 pf0[2], pf1[2];
-        float corr0, corr1;
-        const bool all_visible = wave_rows == 32 &&
-                                 page_fully_visible(wave_first_pos, wave_last_pos, key0, window, sinks);
-        if (all_visible) {
-            softmax_page<false, 16, 4, HD>(s0, st0, scale_log2, q_pos0, key0, window, sinks, pf0, corr0);
-            softmax_page<false, 16, 4, HD>(s1, st1, scale_log2, q_pos1, key0, window, sinks, pf1, corr1);
-        } else {
-            softmax_page<true, 16, 4, HD>(s0, st0, scale_log2, q_pos0, key0, window, sinks, pf0, corr0);
-            softmax_page<true, 16, 4, HD>(s1, st1, scale_log2, q_pos1, key0, window, sinks, pf1, corr1);
-        }
-        const bool rescale = __ballot(corr0 != 1.0f || corr1 != 1.0f) != 0;
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int db = 0; db < HD / 16; ++db) {
-            if (db + kEarly < HD / 16) {
-                vf[db + kEarly][0] = read_v(db + kEarly, 0);
-                vf[db + kEarly][1] = read_v(db + kEarly, 1);
-            }
-            f32x4 a0 = st0.acc[db], a1 = st1.acc[db];
-            if (rescale) {
-#pragma unroll
-                for (int r = 0; r < 4; ++r) { a0[r] *= corr0; a1[r] *= corr1; }
-            }
-#pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                a0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[db][t], pf0[t], a0, 0, 0, 0);
-                a1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[db][t], pf1[t], a1, 0, 0, 0);
-            }
-            st0.acc[db] = a0;
-            st1.acc[db] = a1;
-        }
-        } while (0);
-        land(nxt, lds[buf ^ 1]);
-        cur = nxt;
-        nxt = nxt2;
-        nxt_id = nxt2_id;
-        buf ^= 1;
-        lead = advance(lead);
-    }
-    if (HALVES == 2) {
-        // The second set's running maxima, sums and outputs go through LDS (lane by lane: the two
-        // sets hold the same rows in the same lanes) and are added to the first set's.  The loop's
-        // last barrier came after the last read of a page.
-        constexpr int kStateFloats = 2 + HD / 4;
-        float* state = reinterpret_cast<float*>(smem_raw) + (size_t)wave * (2 * kStateFloats * kWave) + lane;
-        auto put = [&](const WaveState<HD>& st, float* at) {
-            at[0] = st.m;
-            at[kWave] = st.l;
-#pragma unroll
-            for (int db = 0; db < HD / 16; ++db)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) at[(2 + 4 * db + r) * kWave] = st.acc[db][r];
-        };
-        auto add = [&](WaveState<HD>& st, const float* at) {
-            const float m_other = at[0], l_other = at[kWave];
-            const float m = fmaxf(st.m, m_other);
-            const float mine = st.m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(st.m - m);
-            const float theirs = m_other == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_other - m);
-            st.l = st.l * mine + l_other * theirs;
-            st.m = m;
-#pragma unroll
-            for (int db = 0; db < HD / 16; ++db)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) st.acc[db][r] = st.acc[db][r] * mine + at[(2 + 4 * db + r) * kWave] * theirs;
-        };
-        if (set == 1) {
-            put(st0, state);
-            put(st1, state + kStateFloats * kWave);
-        }
-        __syncthreads();
-        if (set == 1) return;
-        add(st0, state);
-        add(st1, state + kStateFloats * kWave);
-    }
-    auto write_out = [&](const WaveState<HD>& st, int rr) {
-        if (rr >= wave_rows) return;
-        const float inv = st.l > 0.f ? 1.0f / st.l : 0.f;
-        bf16_t* orow = out + ((size_t)(row0 + rr) * n_heads + h) * HD;
-#pragma unroll
-        for (int db = 0; db < HD / 16; ++db) {
-            uint2 u;
-            u.x = pack_bf16(st.acc[db][0] * inv, st.acc[db][1] * inv);
-            u.y = pack_bf16(st.acc[db][2] * inv, st.acc[db][3] * inv);
-            *reinterpret_cast<uint2*>(orow + 16 * db + 4 * g) = u;
-        }
-    };
-    write_out(st0, c);
-    write_out(st1, 16 + c);
-}
-
 // ---------------------------------------------------------------- entry points
 static bool mfma_shape_ok(int n_heads, int n_kv_heads, int head_dim) {
     if (n_kv_heads <= 0 || n_heads % n_kv_heads) return false;

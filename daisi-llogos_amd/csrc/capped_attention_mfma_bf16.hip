@@ -14,60 +14,7 @@
 //            (max, sum, output) for a small merge kernel.
 // The sink and the gate are applied where a row is finished (a block's own write, or the merge).
 #include "attention_mfma.h"
-
-// Softmax of one page with the score's scale and bend applied first, in place of softmax_page
-// (which folds a plain scale into its exponent).  y = bend(s * scale) * log2(e); the tanh is
-// 1 - 2 / (exp(2 x) + 1), with the hardware's exp2 and reciprocal.
-template <bool MASKED, int VP>
-__device__ __forceinline__ void softmax_page_bent(f32x4 (&s)[4], WaveState<VP>& st, float scale, float cap, int q_pos,
-                                                  int key0, bf16x8 (&pf)[2], float& corr) {
-    const int g = (threadIdx.x & (kWave - 1)) >> 4;
-    float y[16];
-    if (cap > 0.f) {
-        // cap * tanh(x / cap) * log2(e) = a - 2 a / (exp2(s * b) + 1) with a = cap * log2(e), b = 2 scale log2(e) / cap
-        const float a = cap * kLog2e, b2 = 2.0f * scale * kLog2e / cap;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const float t = __builtin_amdgcn_exp2f(s[i >> 2][i & 3] * b2);
-            y[i] = fmaf(-2.0f * a, __builtin_amdgcn_rcpf(t + 1.0f), a);
-        }
-    } else {
-        const float b1 = scale * kLog2e;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) y[i] = s[i >> 2][i & 3] * b1;
-    }
-    float tile_max = -INFINITY;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        if (MASKED) {
-            const int key = key0 + g * 16 + i;                 // (i = 4 rb + r: the lane's keys are 16 in a row)
-            if (!(q_pos >= 0 && key <= q_pos)) y[i] = -INFINITY;
-        }
-        tile_max = fmaxf(tile_max, y[i]);
-    }
-    tile_max = quad_max(tile_max);
-    const float m_new = fmaxf(st.m, tile_max);
-    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-    corr = __builtin_amdgcn_exp2f(st.m - m_use);
-    float sum = 0.f;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        y[i] = __builtin_amdgcn_exp2f(y[i] - m_use);
-        sum += y[i];
-    }
-    sum = quad_sum(sum);
-    st.l = st.l * corr + sum;
-    st.m = m_new;
-#pragma unroll
-    for (int t = 0; t < 2; ++t) {
-        uint4 u;
-        u.x = pack_bf16(y[8 * t + 0], y[8 * t + 1]);
-        u.y = pack_bf16(y[8 * t + 2], y[8 * t + 3]);
-        u.z = pack_bf16(y[8 * t + 4], y[8 * t + 5]);
-        u.w = pack_bf16(y[8 * t + 6], y[8 * t + 7]);
-        pf[t] = __builtin_bit_cast(bf16x8, u);
-    }
-}
+#include <algorithm>
 
 template <int KP, int VP>
 __device__ __forceinline__ void attend_page_kv(WaveState<VP>& st, const bf16x8 (&qf)[KP / 32], const bf16_t* __restrict__ kpage,
@@ -104,15 +51,6 @@ __device__ __forceinline__ void load_values_kept(bf16x8 (&vf)[VP / 16][2], const
         vf[db][0] = ld_frag(mine + 512 * (2 * db));
         vf[db][1] = ld_frag(mine + 512 * (2 * db + 1));
     }
-}
-
-// What finishes a row: the sink's share of the denominator (exp(0 - max), the maximum being in units of
-// log2) and the head's gate.  Returns the factor on the unnormalised output.
-__device__ __forceinline__ float finish_factor(float m, float l, int unit_sink, const float* gate_logit) {
-    if (unit_sink) l += __builtin_amdgcn_exp2f(-m);
-    float f = l > 0.f ? 1.0f / l : 0.f;
-    if (gate_logit) f *= 1.0f / (1.0f + expf(-*gate_logit));
-    return f;
 }
 
 // ---------------------------------------------------------------- prefill
@@ -320,17 +258,39 @@ static int capped_pages_per_wave(int batch, int n_kv_heads, int table_width) {
     else if (dk == 96 && dv == 96) DO(3, 6); else if (dk == 96 && dv == 128) DO(3, 8); else if (dk == 128 && dv == 64) DO(4, 4); \
     else if (dk == 128 && dv == 80) DO(4, 5); else if (dk == 128 && dv == 96) DO(4, 6); else DO(4, 8);
 
-// -2: a shape these kernels do not take (the caller uses the kernel for any shape).  n_tiles counts tiles of 64
-// rows over all sequences.
+// -2: a shape these kernels do not take (the caller uses the kernel for any shape).  tile_rows 64: the simple form;
+// 128: pages shared through LDS, with one or two sets of waves (`halves`); n_tiles counts tiles of that many rows.
 LLOGOS_EXPORT int llogos_capped_attn_prefill_bf16(void* out, const void* q, int q_stride, const void* k_pool, const void* v_pool,
                                                   const int* table, int table_stride, const int* cu, const int* tok_pos,
                                                   int batch, int n_tiles, int n_heads, int n_kv_heads, int dk, int dv, float scale,
                                                   float softcap, int unit_sink, const float* gate, int gate_stride,
-                                                  hipStream_t stream) {
+                                                  int tile_rows, int halves, hipStream_t stream) {
     if (batch <= 0 || n_tiles <= 0 || softcap < 0.f || (gate && gate_stride < n_heads)) return LLOGOS_BAD_ARGUMENT;
+    if ((tile_rows != 64 && tile_rows != kTileRows) || (halves != 1 && halves != 2)) return LLOGOS_BAD_ARGUMENT;
     if (!capped_shape_ok(n_heads, n_kv_heads, dk, dv) || q_stride % 8) return LLOGOS_UNSUPPORTED;
     dim3 grid(n_tiles, n_heads);
     const int group = n_heads / n_kv_heads;
+    if (tile_rows == kTileRows) {
+        // tiles of 128 tokens whose pages go straight into LDS, once for a block's waves (attention_mfma.h)
+        const long long pairs = (long long)n_tiles * n_kv_heads;
+        const dim3 lgrid((unsigned)((pairs + 7) / 8 * 8 * group));
+#define DIRECT(KS, VB, HALVES) do { \
+        size_t smem = HALVES * 2 * sizeof(DirectPageLds<32 * KS, 16 * VB>); \
+        if (HALVES == 2) smem = std::max(smem, (size_t)kAttnWaves * 2 * (2 + 4 * VB) * kWave * sizeof(float)); \
+        hipError_t e = hipFuncSetAttribute((const void*)attn_prefill_direct_kernel<32 * KS, HALVES, 16 * VB, true>, \
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem); \
+        if (e != hipSuccess) return (int)e; \
+        attn_prefill_direct_kernel<32 * KS, HALVES, 16 * VB, true><<<lgrid, HALVES * kAttnWaves * kWave, smem, stream>>>( \
+            (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, table, table_stride, \
+            cu, tok_pos, batch, n_tiles, n_heads, n_kv_heads, group, scale, 0, 0, softcap, unit_sink, gate, gate_stride); \
+        return LLOGOS_LAUNCH_CHECK(); } while (0)
+#define DIRECT1(KS, VB) DIRECT(KS, VB, 1)
+#define DIRECT2(KS, VB) DIRECT(KS, VB, 2)
+        if (halves == 2) { CAPPED_SHAPES(DIRECT2) } else { CAPPED_SHAPES(DIRECT1) }
+#undef DIRECT2
+#undef DIRECT1
+#undef DIRECT
+    }
 #define PRE(KS, VB) capped_prefill_kernel<KS, VB><<<grid, kAttnWaves * kWave, 0, stream>>>((bf16_t*)out, (const bf16_t*)q, q_stride, \
         (const bf16_t*)k_pool, (const bf16_t*)v_pool, table, table_stride, cu, tok_pos, batch, n_heads, n_kv_heads, group, scale, \
         softcap, unit_sink, gate, gate_stride)

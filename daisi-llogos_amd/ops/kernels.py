@@ -1615,6 +1615,10 @@ def attention(ctx, q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool:
                              n_heads, n_kv_heads, head_dim, scale, window, sinks)
 
 
+CAPPED_PREFILL_TILE_ROWS = 0      # 0: chosen by the step; 64 or 128 force a prompt kernel of the attention with bent scores (tests)
+CAPPED_PREFILL_HALVES = 0         # 0: chosen by the step; 1 or 2 sets of waves a block of the 128-row kernel (tests)
+
+
 def capped_attention(ctx, q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, table: torch.Tensor, n_heads: int,
                      n_kv_heads: int, head_dim: int, v_dim: int, scale: float, softcap: float = 0.0,
                      unit_sink: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -1649,11 +1653,16 @@ def capped_attention(ctx, q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.T
             else:
                 cu = ctx.cu_dev
                 _need(cu is not None and cu.numel() == ctx.batch + 1, "attention: the step's token offsets are missing")
-                n_tiles = sum(-(-(ctx.cu_seqlens[i + 1] - ctx.cu_seqlens[i]) // 64) for i in range(ctx.batch))
+                # long sequences: tiles of 128 tokens whose pages go straight into LDS once for a block's waves (the
+                # dense decoder's prompt kernel with the bent softmax); short ones: tiles of 64 whose waves read the pages
+                lens = [ctx.cu_seqlens[i + 1] - ctx.cu_seqlens[i] for i in range(ctx.batch)]
+                tile_rows = CAPPED_PREFILL_TILE_ROWS or (128 if max(lens) > 64 else 64)
+                n_tiles = sum(-(-n // tile_rows) for n in lens)
+                halves = CAPPED_PREFILL_HALVES or (prefill_halves(lens, getattr(ctx, "starts", None), n_heads) if tile_rows == 128 else 1)
                 code = lib.llogos_capped_attn_prefill_bf16(
                     _p(out), _p(q), q.stride(0), _p(k_pool), _p(v_pool), _p(table), table.stride(0), _p(cu), _p(ctx.tok_pos),
                     ctx.batch, n_tiles, n_heads, n_kv_heads, head_dim, v_dim, ctypes.c_float(scale), ctypes.c_float(softcap),
-                    sink, _p(gate), gate_stride, _stream())
+                    sink, _p(gate), gate_stride, int(tile_rows), int(halves), _stream())
             if code != -2:
                 _check(code, "capped_attention")
                 return out

@@ -170,13 +170,16 @@ def _plain_mixer(mix, plain, h, form):
     return pz.mixer("attention_2" if form == "second" else "attention", m, plain, "m.", h, mix.eps)
 
 
-@pytest.mark.parametrize("dtype", H.DTYPES)
+@pytest.mark.parametrize("dtype,tile_rows,halves", [("float32", 0, 0), ("bfloat16", 0, 0), ("bfloat16", 64, 1), ("bfloat16", 128, 1),
+                                                    ("bfloat16", 128, 2)])
 @pytest.mark.parametrize("shape", MIXERS)
-def test_the_attention_alone_in_pieces(dtype, shape, monkeypatch):
+def test_the_attention_alone_in_pieces(dtype, tile_rows, halves, shape, monkeypatch):
     """Three sequences cut into steps of several sizes, their pages in any order, a page of NaN that nobody
     may read; queries and keys scaled so that single keys decide.  Shapes that the matrix-core kernels
     take must run there in bfloat16."""
     heads, kv, dk, dv, hidden, form = shape
+    monkeypatch.setattr(K, "CAPPED_PREFILL_TILE_ROWS", tile_rows)        # every prompt kernel of the matrix cores in turn
+    monkeypatch.setattr(K, "CAPPED_PREFILL_HALVES", halves)
     rng = np.random.default_rng(heads * 100 + dk)
     mix = _capped(*shape)
     plain = _bind(mix, rng, dtype, scaled={"m.q": 2.0, "m.k": 2.0})
